@@ -1,0 +1,248 @@
+"""CPU oracle for the fused GRPO loss path.  TEST INFRASTRUCTURE ONLY.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import
+this module; the product package never does.
+
+It restates, on flattened tokens and in float64 NumPy, the arithmetic of the
+reference's un-fused jnp loss:
+
+  MLLM_JAX/train_modules/__init__.py:118-192   (logp, entropy, ratio/clip, loss)
+  MLLM_JAX/language/qwen2/modular_qwen2.py:182 (logits = hidden @ lm_head[H,V])
+  deprecated/MLLM_JAX/language/gemma/transformer.py:337-339 (final-logit softcap)
+  plugins/training/update/train_step.py:15-24  (value_and_grad -> closed-form backward)
+  plugins/training/advantage/grpo.py:28-52     (group-normalised advantages)
+  plugins/training/ppo/module.py:59-150        (actor-critic twin; policy part)
+  plugins/sft/jax/sft_module.py:22-45          (masked cross-entropy)
+
+The arithmetic itself lives in un-vendored JAX (jax.nn.log_softmax, jax.nn.softmax,
+jnp.take_along_axis, jnp.clip, jnp.minimum, jax.value_and_grad; version unpinned in
+the reference's requirements-tpu.txt:8-20, docs name jax 0.8.2).  JAX is not
+installable here, and the reference holds no golden vector for this path, so the
+restatement is pinned by what the mathematics fixes (tests/test_oracle_*.py):
+scipy.special.log_softmax/logsumexp, closed forms (uniform logits, on-policy loss),
+the six clip regions enumerated by hand, torch.autograd in float64 and central
+finite differences for the backward, softcap limits, permutation invariance.
+
+Parity unpinned (documented, accepted):
+  * XLA's bf16 rounding of logits under the Qwen dtype policy
+    (modular_qwen2.py:143, llama.py:255-256) is deliberately not replicated: the
+    oracle keeps float64 logits of bf16-valued inputs.
+  * JAX's half-gradient tie rule exactly at ratio == 1-eps_low / 1+eps_high
+    (lax.min / lax.clip JVP); the closed form here takes the full unclipped
+    gradient on the closed interval.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+
+# --------------------------------------------------------------------------- logits
+def lm_head_logits(hidden, lm_head, softcap=None):
+    """z = hidden[N,H] @ lm_head[H,V] (modular_qwen2.py:182), optional
+    z = cap*tanh(z/cap) (gemma/transformer.py:337-339).  float64."""
+    z = np.asarray(hidden, np.float64) @ np.asarray(lm_head, np.float64)
+    if softcap:
+        z = float(softcap) * np.tanh(z / float(softcap))
+    return z
+
+
+def _logsumexp(z):
+    m = z.max(axis=-1, keepdims=True)
+    return (m + np.log(np.exp(z - m).sum(axis=-1, keepdims=True)))[..., 0]
+
+
+# --------------------------------------------------------------------------- forward
+def token_logps_and_entropy(z, target_ids, temperature=1.0):
+    """train_modules/__init__.py:124-126 and :136-138 on logits z[N,V].
+
+    logp  = log_softmax(z)[t, y_t] / T        (division AFTER the log-softmax)
+    probs = softmax(z / T);  H_t = -sum(probs * log(probs + 1e-9))
+    Returns (logp[N], lse[N], token_entropy[N])."""
+    z = np.asarray(z, np.float64)
+    n = z.shape[0]
+    y = np.asarray(target_ids).astype(np.int64)
+    lse = _logsumexp(z)
+    logp = (z[np.arange(n), y] - lse) / float(temperature)
+    zt = z / float(temperature)
+    p = np.exp(zt - _logsumexp(zt)[:, None])
+    ent = -(p * np.log(p + 1e-9)).sum(axis=-1)
+    return logp, lse, ent
+
+
+def sequence_entropy_stats(token_entropy, mask, seq_shape):
+    """train_modules/__init__.py:141-157: per-sample masked mean entropy and the
+    'tokens 4..100 of the completion' truncated mean.  Empty rows give nan (the
+    reference divides by zero there too)."""
+    b, t = seq_shape
+    ent = np.asarray(token_entropy, np.float64).reshape(b, t)
+    m = np.asarray(mask).reshape(b, t)
+    mf = m.astype(np.float64)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        avg = (ent * mf).sum(-1) / mf.sum(-1)
+        valid = (m == 1)
+        cum = np.cumsum(valid, axis=-1)
+        win = valid & (cum >= 4) & (cum <= 100)
+        avg_trunc = (ent * win).sum(-1) / win.sum(-1)
+    return avg, avg_trunc
+
+
+def policy_loss_terms(logp, old_logp, advantages, mask, total_valid_token_count,
+                      eps_low, eps_high):
+    """train_modules/__init__.py:161-180.  Returns (loss, dloss/dlogp[N]).
+
+    ratio = exp(logp-old); clipped = clip(ratio, 1-eps_low, 1+eps_high)
+    loss  = sum(-min(ratio*adv, clipped*adv) * mask) / tvtc
+    d/dlogp: -(mask/tvtc)*adv*ratio where the unclipped branch is the active min
+    (inside the interval always; above it only for adv<0; below it only for adv>0)."""
+    logp = np.asarray(logp, np.float64)
+    old = logp if old_logp is None else np.asarray(old_logp, np.float64)
+    adv = np.asarray(advantages, np.float64)
+    m = np.asarray(mask, np.float64)
+    lo, hi = 1.0 - float(eps_low), 1.0 + float(eps_high)
+    ratio = np.exp(logp - old)
+    clipped = np.clip(ratio, lo, hi)
+    ptl = -np.minimum(ratio * adv, clipped * adv)
+    tv = float(m.sum()) if total_valid_token_count is None else float(total_valid_token_count)
+    loss = (ptl * m).sum() / tv
+    active = ((ratio >= lo) & (ratio <= hi)) | ((ratio > hi) & (adv < 0)) | ((ratio < lo) & (adv > 0))
+    g = -(m / tv) * adv * ratio * active
+    return loss, g
+
+
+def grpo_loss(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
+              total_valid_token_count=None, epsilon_low=0.2, epsilon_high=0.3,
+              temperature=1.0, final_logit_softcap=None, seq_shape=None,
+              with_grads=True):
+    """Whole path, float64.  Mirrors TrainGRPOModule.__call__'s return dict
+    (train_modules/__init__.py:185-192) plus token_entropy/lse and, when asked, the
+    closed-form gradients d_hidden[N,H], d_lm_head[H,V] that jax.value_and_grad
+    (update/train_step.py:24) yields for the loss."""
+    h = np.asarray(hidden, np.float64)
+    w = np.asarray(lm_head, np.float64)
+    n = h.shape[0]
+    y = np.asarray(target_ids).astype(np.int64)
+    z_raw = h @ w
+    cap = float(final_logit_softcap) if final_logit_softcap else None
+    z = cap * np.tanh(z_raw / cap) if cap else z_raw
+    logp, lse, ent = token_logps_and_entropy(z, y, temperature)
+    adv = np.asarray(advantages, np.float64)
+    if seq_shape is not None and adv.shape[0] == seq_shape[0] and adv.shape[0] != n:
+        adv = np.repeat(adv, seq_shape[1])          # [B] -> [B,1] broadcast, :173
+    loss, g = policy_loss_terms(logp, old_logps, adv, mask, total_valid_token_count,
+                                epsilon_low, epsilon_high)
+    out = {"loss": loss, "per_token_logps": logp, "lse": lse, "token_entropy": ent}
+    if seq_shape is not None:
+        out["entropy"], out["entropy_loss"] = sequence_entropy_stats(ent, mask, seq_shape)
+    if with_grads:
+        p = np.exp(z - lse[:, None])
+        dz = -p
+        dz[np.arange(n), y] += 1.0
+        dz *= (g / float(temperature))[:, None]
+        if cap:
+            dz *= 1.0 - (z / cap) ** 2              # d tanh = 1 - tanh^2
+        out["d_hidden"] = dz @ w.T
+        out["d_lm_head"] = h.T @ dz
+        out["dlogp"] = g
+    return out
+
+
+# --------------------------------------------------------------------------- siblings
+def grpo_advantages(rewards, group_ids, eps=1e-4):
+    """plugins/training/advantage/grpo.py:28-52: (r - mean_g) / (std_g + eps),
+    population std, float32 result."""
+    r = np.asarray(rewards, np.float32)
+    _, inv = np.unique(np.asarray(group_ids), return_inverse=True)
+    ng = int(inv.max()) + 1
+    cnt = np.maximum(np.bincount(inv, minlength=ng).astype(np.float32), 1.0)
+    mean = np.bincount(inv, weights=r, minlength=ng).astype(np.float32) / cnt
+    c = r - mean[inv]
+    std = np.sqrt(np.bincount(inv, weights=c * c, minlength=ng).astype(np.float32) / cnt)
+    return (c / (std[inv] + float(eps))).astype(np.float32)
+
+
+def sft_cross_entropy(hidden, lm_head, labels, valid, *, with_grads=True):
+    """plugins/sft/jax/sft_module.py:22-45 on flattened, already shifted tokens:
+    loss = sum(-log_softmax(z)[t,label_t] * valid) / max(sum(valid), 1)."""
+    h = np.asarray(hidden, np.float64)
+    w = np.asarray(lm_head, np.float64)
+    v = np.asarray(valid, np.float64)
+    y = np.where(np.asarray(valid).astype(bool), np.asarray(labels), 0).astype(np.int64)
+    n = h.shape[0]
+    z = h @ w
+    lse = _logsumexp(z)
+    logp = z[np.arange(n), y] - lse
+    denom = max(float(v.sum()), 1.0)
+    out = {"loss": (-logp * v).sum() / denom, "token_count": int(v.sum()), "per_token_logps": logp}
+    if with_grads:
+        dz = np.exp(z - lse[:, None])
+        dz[np.arange(n), y] -= 1.0
+        dz *= (v / denom)[:, None]
+        out["d_hidden"] = dz @ w.T
+        out["d_lm_head"] = h.T @ dz
+    return out
+
+
+# ------------------------------------------------------------- large-shape oracle (torch)
+def grpo_loss_chunked_torch(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
+                            total_valid_token_count=None, epsilon_low=0.2, epsilon_high=0.3,
+                            final_logit_softcap=None, with_grads=True, chunk=1024,
+                            dtype=None, rows=None):
+    """Same arithmetic as grpo_loss (temperature 1) in torch on the CPU, token-chunked
+    so BASELINE-sized shapes fit in host memory.  float32 matmul by default (inputs are
+    bf16-valued, so products are exact and only the accumulation rounds), float64
+    softmax statistics.  `rows` restricts the work to a subset of token rows while the
+    normaliser stays that of the whole batch; d_lm_head is then that subset's share."""
+    import torch
+
+    dt = dtype or torch.float32
+    h = torch.as_tensor(hidden).to(dt)
+    w = torch.as_tensor(lm_head).to(dt)
+    y = torch.as_tensor(target_ids).long()
+    adv = torch.as_tensor(advantages).double()
+    m = torch.as_tensor(mask).double()
+    n = h.shape[0]
+    tv = float(m.sum()) if total_valid_token_count is None else float(total_valid_token_count)
+    old = None if old_logps is None else torch.as_tensor(old_logps).double()
+    idx = torch.arange(n) if rows is None else torch.as_tensor(rows).long()
+    cap = float(final_logit_softcap) if final_logit_softcap else None
+    lo, hi = 1.0 - float(epsilon_low), 1.0 + float(epsilon_high)
+    logp = torch.zeros(n, dtype=torch.float64)
+    lse = torch.zeros(n, dtype=torch.float64)
+    ent = torch.zeros(n, dtype=torch.float64)
+    ptl = torch.zeros(n, dtype=torch.float64)
+    d_h = torch.zeros(h.shape, dtype=torch.float32) if with_grads else None
+    d_w = torch.zeros(w.shape, dtype=torch.float32) if with_grads else None
+    for s in range(0, idx.numel(), chunk):
+        r = idx[s:s + chunk]
+        z = (h[r] @ w).double()
+        if cap:
+            z = cap * torch.tanh(z / cap)
+        l = torch.logsumexp(z, dim=-1)
+        zy = z.gather(1, y[r, None])[:, 0]
+        lp = zy - l
+        p = torch.exp(z - l[:, None])
+        e = -(p * torch.log(p + 1e-9)).sum(-1)
+        o = lp if old is None else old[r]
+        ratio = torch.exp(lp - o)
+        clipped = ratio.clamp(lo, hi)
+        a = adv[r]
+        ptl[r] = -torch.minimum(ratio * a, clipped * a)
+        logp[r], lse[r], ent[r] = lp, l, e
+        if with_grads:
+            active = ((ratio >= lo) & (ratio <= hi)) | ((ratio > hi) & (a < 0)) | ((ratio < lo) & (a > 0))
+            g = -(m[r] / tv) * a * ratio * active
+            dz = -p
+            dz.scatter_add_(1, y[r, None], torch.ones(len(r), 1, dtype=torch.float64))
+            dz *= g[:, None]
+            if cap:
+                dz *= 1.0 - (z / cap) ** 2
+            dzf = dz.to(dt)
+            d_h[r] = (dzf @ w.T).float()
+            d_w += (h[r].T @ dzf).float()
+    loss = float((ptl * m).sum() / tv)
+    out = {"loss": loss, "per_token_logps": logp.numpy(), "lse": lse.numpy(),
+           "token_entropy": ent.numpy()}
+    if with_grads:
+        out["d_hidden"] = d_h.numpy()
+        out["d_lm_head"] = d_w.numpy()
+    return out

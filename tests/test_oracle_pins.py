@@ -1,0 +1,230 @@
+"""Pins the CPU oracle (oracle/grpo_oracle.py) against what the mathematics fixes.
+
+The reference holds no golden vector for this path (its tests never touch
+TrainGRPOModule), so every check here is independent of the oracle's own formula:
+scipy/torch library routines, closed forms, hand-enumerated clip regions, float64
+autograd and central finite differences.
+"""
+import numpy as np
+import pytest
+import scipy.special as sps
+import torch
+
+from oracle import grpo_oracle as O
+
+
+def _inputs(rng, n=12, h=8, v=37, b=3):
+    hid = rng.standard_normal((n, h))
+    w = rng.standard_normal((h, v)) * 0.5
+    y = rng.integers(0, v, n)
+    adv = np.repeat(rng.standard_normal(b), n // b)
+    lens = rng.integers(1, n // b + 1, b)
+    mask = (np.arange(n // b)[None, :] < lens[:, None]).astype(np.float64).reshape(-1)
+    return hid, w, y, adv, mask
+
+
+def test_logp_matches_scipy_log_softmax(rng):
+    hid, w, y, *_ = _inputs(rng)
+    z = hid @ w
+    logp, lse, _ = O.token_logps_and_entropy(z, y)
+    np.testing.assert_allclose(lse, sps.logsumexp(z, axis=-1), rtol=0, atol=1e-12)
+    np.testing.assert_allclose(logp, sps.log_softmax(z, axis=-1)[np.arange(len(y)), y], atol=1e-12)
+
+
+def test_temperature_divides_after_log_softmax(rng):
+    # reference quirk: log_softmax(z)[y] / T, but entropy of softmax(z / T)
+    hid, w, y, *_ = _inputs(rng)
+    z = hid @ w
+    lp1, _, _ = O.token_logps_and_entropy(z, y, 1.0)
+    lp2, _, e2 = O.token_logps_and_entropy(z, y, 2.0)
+    np.testing.assert_allclose(lp2, lp1 / 2.0, atol=1e-13)
+    p = sps.softmax(z / 2.0, axis=-1)
+    np.testing.assert_allclose(e2, -(p * np.log(p + 1e-9)).sum(-1), atol=1e-12)
+
+
+def test_uniform_logits_closed_form():
+    v = 151936
+    z = np.zeros((3, v))
+    logp, lse, ent = O.token_logps_and_entropy(z, np.array([0, 5, v - 1]))
+    np.testing.assert_allclose(logp, -np.log(v), atol=1e-12)
+    np.testing.assert_allclose(lse, np.log(v), atol=1e-12)
+    # -sum p log(p+1e-9) with p = 1/V
+    np.testing.assert_allclose(ent, -np.log(1.0 / v + 1e-9), atol=1e-9)
+    assert abs(ent[0] - np.log(v)) <= v * 1e-9
+
+
+def test_dominant_logit_limit():
+    z = np.full((1, 50), -40.0)
+    z[0, 7] = 40.0
+    logp, _, ent = O.token_logps_and_entropy(z, np.array([7]))
+    assert abs(logp[0]) < 1e-12 and abs(ent[0]) < 1e-6
+
+
+def test_stream_entropy_bound(rng):
+    # lse - sum p z differs from the reference's -sum p log(p+1e-9) by at most V*1e-9
+    hid, w, y, *_ = _inputs(rng, v=296)
+    z = hid @ w
+    _, lse, ent = O.token_logps_and_entropy(z, y)
+    p = sps.softmax(z, axis=-1)
+    stream = lse - (p * z).sum(-1)
+    assert np.all(stream - ent >= -1e-12) and np.all(stream - ent <= 296 * 1e-9)
+
+
+@pytest.mark.parametrize("eps", [(0.2, 0.2), (0.2, 0.28), (0.2, 0.3)])
+def test_clip_regions_by_hand(eps):
+    lo, hi = 1 - eps[0], 1 + eps[1]
+    ratios = np.array([0.5, 0.9, 1.0, 1.25, 1.29, 2.0])
+    for adv in (-1.0, 1.0):
+        logp = np.zeros(6)
+        old = -np.log(ratios)
+        loss, g = O.policy_loss_terms(logp, old, np.full(6, adv), np.ones(6), 6.0, *eps)
+        exp_terms, exp_g = [], []
+        for r in ratios:
+            if adv > 0:       # A*min(r, clip(r)): capped above
+                val = adv * min(r, hi)
+                grad_on = r <= hi
+            else:             # A*max(r, clip(r)): floored below
+                val = adv * max(r, lo)
+                grad_on = r >= lo
+            exp_terms.append(-val)
+            exp_g.append(-(adv * r) / 6.0 if grad_on else 0.0)
+        np.testing.assert_allclose(loss, np.sum(exp_terms) / 6.0, atol=1e-12)
+        np.testing.assert_allclose(g, exp_g, atol=1e-12)
+
+
+def test_on_policy_closed_form(rng):
+    hid, w, y, adv, mask = _inputs(rng)
+    out = O.grpo_loss(hid, w, y, None, adv, mask, seq_shape=(3, 4))
+    tv = mask.sum()
+    np.testing.assert_allclose(out["loss"], -(adv * mask).sum() / tv, atol=1e-12)
+    p = sps.softmax(hid @ w, axis=-1)
+    onehot = np.eye(w.shape[1])[y]
+    dz = (-(mask * adv) / tv)[:, None] * (onehot - p)
+    np.testing.assert_allclose(out["d_hidden"], dz @ w.T, atol=1e-12)
+    np.testing.assert_allclose(out["d_lm_head"], hid.T @ dz, atol=1e-12)
+
+
+def test_mask_tvtc_and_zero_adv(rng):
+    hid, w, y, adv, mask = _inputs(rng)
+    old = O.grpo_loss(hid, w, y, None, adv, mask)["per_token_logps"] + 0.05 * rng.standard_normal(12)
+    a = O.grpo_loss(hid, w, y, old, adv, mask, total_valid_token_count=7.0)
+    b = O.grpo_loss(hid, w, y, old, adv, mask, total_valid_token_count=14.0)
+    np.testing.assert_allclose(b["loss"], a["loss"] / 2, rtol=1e-13)
+    np.testing.assert_allclose(b["d_lm_head"], a["d_lm_head"] / 2, rtol=1e-12, atol=1e-15)
+    assert np.all(a["d_hidden"][mask == 0] == 0)
+    z = O.grpo_loss(hid, w, y, old, np.zeros(12), mask)
+    assert z["loss"] == 0 and not z["d_hidden"].any() and not z["d_lm_head"].any()
+
+
+def _torch_twin(hid, w, y, old, adv, mask, tv, eps, cap, T=1.0):
+    h = torch.tensor(hid, dtype=torch.float64, requires_grad=True)
+    ww = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+    z = h @ ww
+    if cap:
+        z = torch.tanh(z / cap) * cap
+    lp = torch.log_softmax(z, -1).gather(1, torch.tensor(y)[:, None])[:, 0] / T
+    o = lp.detach() if old is None else torch.tensor(old)
+    r = torch.exp(lp - o)
+    a = torch.tensor(adv)
+    ptl = -torch.minimum(r * a, r.clamp(1 - eps[0], 1 + eps[1]) * a)
+    loss = (ptl * torch.tensor(mask)).sum() / tv
+    loss.backward()
+    return loss.item(), lp.detach().numpy(), h.grad.numpy(), ww.grad.numpy()
+
+
+@pytest.mark.parametrize("cap", [None, 30.0, 2.0])
+@pytest.mark.parametrize("T", [1.0, 0.7])
+def test_backward_matches_float64_autograd(rng, cap, T):
+    hid, w, y, adv, mask = _inputs(rng)
+    hid *= 2.0
+    base = O.grpo_loss(hid, w, y, None, adv, mask, final_logit_softcap=cap, temperature=T)
+    old = base["per_token_logps"] + 0.3 * rng.standard_normal(12)   # wide: hits clip regions
+    out = O.grpo_loss(hid, w, y, old, adv, mask, total_valid_token_count=9.0,
+                      epsilon_low=0.2, epsilon_high=0.28, final_logit_softcap=cap, temperature=T)
+    loss, lp, dh, dw = _torch_twin(hid, w, y, old, adv, mask, 9.0, (0.2, 0.28), cap, T)
+    np.testing.assert_allclose(out["loss"], loss, rtol=1e-12)
+    np.testing.assert_allclose(out["per_token_logps"], lp, atol=1e-12)
+    np.testing.assert_allclose(out["d_hidden"], dh, atol=1e-12)
+    np.testing.assert_allclose(out["d_lm_head"], dw, atol=1e-12)
+    assert np.abs(out["d_hidden"]).max() > 0
+
+
+def test_backward_matches_finite_differences(rng):
+    hid, w, y, adv, mask = _inputs(rng, n=6, h=4, v=9, b=3)
+    old = O.grpo_loss(hid, w, y, None, adv, mask)["per_token_logps"] + 0.05 * rng.standard_normal(6)
+    f = lambda hh, ww: O.grpo_loss(hh, ww, y, old, adv, mask, final_logit_softcap=5.0,
+                                   with_grads=False)["loss"]
+    out = O.grpo_loss(hid, w, y, old, adv, mask, final_logit_softcap=5.0)
+    d = 1e-6
+    for (i, j) in [(0, 0), (3, 2), (5, 3)]:
+        e = np.zeros_like(hid); e[i, j] = d
+        np.testing.assert_allclose((f(hid + e, w) - f(hid - e, w)) / (2 * d), out["d_hidden"][i, j], atol=1e-8)
+    for (i, j) in [(0, 0), (2, 8), (3, int(y[0]))]:
+        e = np.zeros_like(w); e[i, j] = d
+        np.testing.assert_allclose((f(hid, w + e) - f(hid, w - e)) / (2 * d), out["d_lm_head"][i, j], atol=1e-8)
+
+
+def test_dz_rows_sum_to_zero_and_softcap_limit(rng):
+    hid, w, y, adv, mask = _inputs(rng)
+    a = O.grpo_loss(hid, w, y, None, adv, mask)
+    b = O.grpo_loss(hid, w, y, None, adv, mask, final_logit_softcap=1e9)
+    np.testing.assert_allclose(a["per_token_logps"], b["per_token_logps"], atol=1e-9)
+    np.testing.assert_allclose(a["d_lm_head"], b["d_lm_head"], atol=1e-9)
+    # d_lm_head = h^T dz and rows of dz sum to zero  =>  d_lm_head @ 1 = 0
+    np.testing.assert_allclose(a["d_lm_head"].sum(-1), 0, atol=1e-12)
+
+
+def test_column_permutation_invariance(rng):
+    hid, w, y, adv, mask = _inputs(rng)
+    perm = rng.permutation(w.shape[1])
+    inv = np.argsort(perm)
+    a = O.grpo_loss(hid, w, y, None, adv, mask)
+    b = O.grpo_loss(hid, w[:, perm], inv[y], None, adv, mask)
+    np.testing.assert_allclose(a["per_token_logps"], b["per_token_logps"], atol=1e-12)
+    np.testing.assert_allclose(a["d_lm_head"][:, perm], b["d_lm_head"], atol=1e-12)
+
+
+def test_sequence_entropy_stats_by_hand():
+    ent = np.arange(1.0, 13.0).reshape(2, 6)
+    mask = np.array([[0, 1, 1, 1, 1, 1], [1, 1, 0, 0, 0, 0]])
+    avg, trunc = O.sequence_entropy_stats(ent.reshape(-1), mask.reshape(-1), (2, 6))
+    np.testing.assert_allclose(avg, [(2 + 3 + 4 + 5 + 6) / 5, (7 + 8) / 2])
+    # window = valid tokens whose running valid count is in [4, 100]
+    np.testing.assert_allclose(trunc[0], (5 + 6) / 2)
+    assert np.isnan(trunc[1])
+
+
+def test_grpo_advantages_closed_form():
+    # advantage/grpo.py:28-52: population std within group, eps 1e-4
+    adv = O.grpo_advantages([1, 0, 0, 0, 1, 1], [7, 7, 7, 7, 9, 9])
+    m, s = 0.25, np.sqrt(0.1875)
+    np.testing.assert_allclose(adv[:4], [(1 - m) / (s + 1e-4)] + [(0 - m) / (s + 1e-4)] * 3, rtol=1e-6)
+    np.testing.assert_allclose(adv[4:], 0.0, atol=1e-7)
+    assert adv.dtype == np.float32
+
+
+def test_sft_cross_entropy_vs_torch(rng):
+    hid, w, y, _, mask = _inputs(rng)
+    out = O.sft_cross_entropy(hid, w, y, mask)
+    h = torch.tensor(hid, requires_grad=True); ww = torch.tensor(w, requires_grad=True)
+    nll = torch.nn.functional.cross_entropy(h @ ww, torch.tensor(y), reduction="none")
+    loss = (nll * torch.tensor(mask)).sum() / max(mask.sum(), 1.0)
+    loss.backward()
+    np.testing.assert_allclose(out["loss"], loss.item(), rtol=1e-12)
+    np.testing.assert_allclose(out["d_lm_head"], ww.grad.numpy(), atol=1e-12)
+    np.testing.assert_allclose(out["d_hidden"], h.grad.numpy(), atol=1e-12)
+
+
+def test_chunked_torch_oracle_matches_float64(rng):
+    hid, w, y, adv, mask = _inputs(rng, n=24, h=16, v=200, b=3)
+    from conftest import bf16_round
+    hid, w = bf16_round(hid), bf16_round(w)
+    old = O.grpo_loss(hid, w, y, None, adv, mask)["per_token_logps"] + 0.05 * rng.standard_normal(24)
+    a = O.grpo_loss(hid, w, y, old, adv, mask, final_logit_softcap=30.0, epsilon_high=0.2)
+    b = O.grpo_loss_chunked_torch(hid, w, y, old, adv, mask, final_logit_softcap=30.0,
+                                  epsilon_high=0.2, chunk=7)
+    np.testing.assert_allclose(b["loss"], a["loss"], rtol=1e-6)
+    np.testing.assert_allclose(b["per_token_logps"], a["per_token_logps"], atol=1e-5)
+    np.testing.assert_allclose(b["token_entropy"], a["token_entropy"], atol=1e-5)
+    np.testing.assert_allclose(b["d_hidden"], a["d_hidden"], atol=1e-6)
+    np.testing.assert_allclose(b["d_lm_head"], a["d_lm_head"], atol=1e-6)
