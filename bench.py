@@ -1,0 +1,132 @@
+"""Benchmark of the fused GRPO loss (forward + backward) on one MI355X.
+
+`python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2]` prints ONE JSON line.
+A step is one fwd+bwd pass of the loss over one synthetic batch of the chosen configuration
+(default: BASELINE.json configs[2], the Qwen2.5-7B shape 16384 x 3584 x 152064 the metric is
+quoted on), inputs resident in HBM, through the host API that wraps the C ABI.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBS = 8000.0
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (profiles/), keyed by (config index, kernel); None until measured for that workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (default 2)")
+    ap.add_argument("--chunk-tokens", type=int, default=0)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the loss path on ONE GPU (no collectives, no sharding); "
+              "run it with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import mllm_jax_amd as M
+    from mllm_jax_amd import _lib
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the fused loss has no CPU path", file=sys.stderr)
+        return 3
+    dev = torch.device("cuda:0")
+    cfg = M.CONFIGS[args.config]
+    kw = dict(epsilon_low=cfg.eps_low, epsilon_high=cfg.eps_high, final_logit_softcap=cfg.softcap,
+              chunk_tokens=args.chunk_tokens or None)
+
+    def logp_fn(wl):
+        with torch.no_grad():
+            out = M.grpo_fused_loss(wl["hidden"], wl["lm_head"], wl["target_ids"], None, wl["advantages"],
+                                    wl["mask"], total_valid_token_count=wl["total_valid_token_count"], **kw)
+        return out["per_token_logps"]
+
+    wl = M.make_workload(cfg, dev, 20250 + args.config, logp_fn=logp_fn)
+    n, h, v = cfg.tokens, cfg.hidden, cfg.vocab
+    d_w = torch.empty(h, v, dtype=torch.float32, device=dev)
+
+    def step():
+        return M.grpo_loss_value_and_grad(
+            wl["hidden"], wl["lm_head"], wl["target_ids"], wl["old_logps"], wl["advantages"], wl["mask"],
+            total_valid_token_count=wl["total_valid_token_count"], seq_shape=wl["seq_shape"],
+            return_token_entropy=cfg.token_entropy, **kw)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.profile_begin(64 * max(args.steps, 1))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        metrics, grads = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    prof = _lib.profile_end()
+    del d_w
+
+    ms_per_step = dt / args.steps * 1e3
+    tokens_per_s = n * args.steps / dt
+    flop_step = 6.0 * n * h * v
+    mfu = flop_step / (ms_per_step * 1e-3) / (PEAK_BF16_TFLOPS * 1e12)
+
+    gemms = {k: prof[k] for k in ("k_logits_stats", "k_dhidden", "k_dw")}
+    dom = max(gemms, key=lambda k: gemms[k][0])
+    dom_ms, dom_launches = gemms[dom]
+    flop_per_launch = 2.0 * n * h * v * args.steps / max(dom_launches, 1)   # algorithmic 2*n_chunk*H*V
+    avg_launch_ms = dom_ms / max(dom_launches, 1)
+    achieved = flop_per_launch / (avg_launch_ms * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+                "avg_launch_ms": round(avg_launch_ms, 3), "launches": dom_launches,
+                "flop_per_launch": flop_per_launch,
+                "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom))}
+
+    line = {
+        "metric": "grpo_fused_loss_fwd_bwd_tokens_per_s", "value": round(tokens_per_s, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"BASELINE configs[{args.config}] {cfg.name}: fused GRPO loss fwd+bwd, "
+                               f"{n} tokens x hidden {h} x vocab {v}", "tokens": n, "hidden": h, "vocab": v,
+                   "chunk_tokens": args.chunk_tokens or 8192, "softcap": cfg.softcap,
+                   "eps": [cfg.eps_low, cfg.eps_high]},
+        "pct_bf16_mfma_peak": round(100.0 * mfu, 2),
+        "algorithmic_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 1),
+        "loss": float(metrics["loss"].item()),
+        "roofline": roofline,
+        "kernel_ms_per_step": {k: round(v_[0] / args.steps, 3) for k, v_ in prof.items()},
+    }
+
+    if not args.no_cpu_baseline:
+        from oracle.cpu_baseline import time_cpu_baseline
+        cpu_wl = {k: (t.cpu() if hasattr(t, "cpu") else t) for k, t in wl.items()}
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        res = time_cpu_baseline(cpu_wl, min(args.cpu_sample_tokens, n), repeats=1, threads=cores)
+        line["cpu_baseline"] = {
+            "value": round(res["tokens_per_s"], 2), "unit": "tokens/s", "cores": res["cores"], "kind": "port",
+            "sample": f"first {res['sample_tokens']} tokens of the same batch at full hidden/vocab, un-fused "
+                      f"float32 torch-CPU fwd+bwd, {res['seconds']:.1f} s (JAX is not installed)"}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,132 @@
+/* mj_grpo.h -- C ABI of the MI355X (gfx950) fused GRPO loss library, libmj_grpo.so.
+ *
+ * The reference (demon2036/MLLM-JAX) has no FFI for this path: the boundary there is
+ * the Python callable TrainGRPOModule.__call__ (MLLM_JAX/train_modules/__init__.py:96-192)
+ * differentiated by jax.value_and_grad (plugins/training/update/train_step.py:15-24).
+ * The entry points below are what a binding for that callable would call; each one
+ * names the reference statements it replaces.
+ *
+ * Conventions: plain pointers to DEVICE memory and sizes, no allocation inside the
+ * library, every kernel is enqueued on the caller's hipStream_t (passed as void*),
+ * calls return immediately (asynchronous), status is an int (0 = ok) and
+ * mj_grpo_last_error() gives the message of the calling thread's last failure.
+ * Two calls may overlap only if they use distinct workspaces.
+ *
+ * Shapes: tokens are flattened, N = B*(L-1) after the reference's shift
+ * (train_modules/__init__.py:118-125).  hidden[N, ld_hidden] bf16 row-major,
+ * lm_head[H, ld_w] bf16 row-major (Flax Dense kernel layout [in, out],
+ * MLLM_JAX/language/llama/llama.py:889), targets[N] int32 in [0, V),
+ * old_logp[N] f32 or NULL (NULL = on-policy, ratio == 1, train_modules/__init__.py:161-165),
+ * advantages[N] f32 (the reference's [B] broadcast per token, :173), mask[N] f32 in {0,1}.
+ * Requirements: H % 8 == 0, V % 8 == 0, ld_hidden % 8 == 0, ld_w % 8 == 0,
+ * bf16 pointers 16-byte aligned, temperature == 1.
+ */
+#ifndef MJ_GRPO_H
+#define MJ_GRPO_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  MJ_GRPO_OK = 0,
+  MJ_GRPO_ERR_NULL = 1,        /* required pointer is NULL */
+  MJ_GRPO_ERR_SHAPE = 2,       /* N/H/V/ld out of range */
+  MJ_GRPO_ERR_ALIGN = 3,       /* pointer or leading dimension not 16-byte aligned */
+  MJ_GRPO_ERR_WORKSPACE = 4,   /* workspace missing or too small */
+  MJ_GRPO_ERR_UNSUPPORTED = 5, /* e.g. temperature != 1 */
+  MJ_GRPO_ERR_HIP = 6          /* a HIP call or kernel launch failed */
+};
+
+enum {
+  MJ_GRPO_FLAG_DW_ACCUMULATE = 1u << 0, /* d_lm_head += (grad accumulation, train_step.py:30-33) */
+  MJ_GRPO_FLAG_SFT = 1u << 1            /* masked cross-entropy instead of the clipped surrogate
+                                           (plugins/sft/jax/sft_module.py:22-45): per-token loss
+                                           -logp, advantages/old_logp ignored */
+};
+
+typedef struct MjGrpoDesc {
+  int64_t n_tokens;      /* N */
+  int64_t hidden;        /* H */
+  int64_t vocab;         /* V */
+  int64_t ld_hidden;     /* elements between rows of hidden (>= H) */
+  int64_t ld_w;          /* elements between rows of lm_head (>= V) */
+  int64_t chunk_tokens;  /* tokens whose 16-bit logits live in the workspace at once; 0 = default */
+  float eps_low;         /* TrainGRPOModule.epsilon_low  (train_modules/__init__.py:92) */
+  float eps_high;        /* TrainGRPOModule.epsilon_high (:93) */
+  float temperature;     /* must be 1 (:91) */
+  float softcap;         /* final-logit softcap, 0 = off (gemma/transformer.py:337-339) */
+  float inv_total_valid_tokens; /* 1 / total_valid_token_count (:179-180) */
+  float grad_loss_scale; /* upstream d(loss); 1 for a terminal loss */
+  uint32_t flags;
+  uint32_t reserved;
+} MjGrpoDesc;
+
+/* Library version, MAJOR*10000 + MINOR*100 + PATCH. */
+int mj_grpo_version(void);
+
+/* Message of the calling thread's last non-zero status ("" if none). */
+const char* mj_grpo_last_error(void);
+
+/* Workspace sizes in bytes for the three entry points below. */
+int mj_grpo_workspace_bytes(const MjGrpoDesc* desc, size_t* forward_bytes,
+                            size_t* forward_backward_bytes);
+
+/* Forward only (no gradient).  Replaces train_modules/__init__.py:124-126 (log-softmax +
+ * gather), :136-138 (per-token entropy), :161-180 (ratio, clip, min, masked normalised sum)
+ * on top of the lm_head product (qwen2/modular_qwen2.py:182), streaming over vocab tiles:
+ * no [N,V] tensor is written.  Outputs: logp[N], lse[N], token_entropy[N] (may be NULL),
+ * loss[1].  */
+int mj_grpo_forward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
+                    const int32_t* targets, const float* old_logp, const float* advantages,
+                    const float* mask, float* logp, float* lse, float* token_entropy,
+                    float* loss, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Forward and backward in one pass (executes 6*N*H*V flop).  Replaces
+ * jax.value_and_grad(loss_fn) of plugins/training/update/train_step.py:15-24 restricted to
+ * the lm_head + loss part: besides the forward outputs it writes
+ * d_hidden[N, ld_hidden] bf16 and d_lm_head[H, ld_w] f32, both already multiplied by
+ * grad_loss_scale.  The workspace holds 16-bit (half) logits for chunk_tokens tokens at a time. */
+int mj_grpo_forward_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
+                             const int32_t* targets, const float* old_logp,
+                             const float* advantages, const float* mask, float* logp,
+                             float* lse, float* token_entropy, float* loss, void* d_hidden,
+                             float* d_lm_head, void* workspace, size_t workspace_bytes,
+                             void* stream);
+
+/* Backward from a saved forward (lse[N], logp[N]): recomputes the logits chunk by chunk
+ * (8*N*H*V flop with the forward).  Same outputs as the backward half above.  For callers
+ * that must separate the two passes (e.g. a forward under no-grad followed later by a
+ * backward with a non-unit upstream gradient). */
+int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
+                     const int32_t* targets, const float* old_logp, const float* advantages,
+                     const float* mask, const float* lse, const float* logp, void* d_hidden,
+                     float* d_lm_head, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Optional per-kernel timing (bench and profiling; no counterpart in the reference, whose only
+ * timers are wall-clock phase timers, plugins/training/runner/grpo_gsm8k.py:615-792).
+ * Between begin and end every kernel launch of the entry points above is bracketed by a pair of
+ * HIP events recorded on the caller's stream.  mj_grpo_profile_end waits for them and returns,
+ * per kernel id, the summed duration in milliseconds and the number of launches.  Process-wide
+ * and not thread-safe: use from one thread. */
+enum {
+  MJ_GRPO_K_TRANSPOSE = 0,
+  MJ_GRPO_K_TARGET_LOGIT = 1,
+  MJ_GRPO_K_LOGITS_STATS = 2,
+  MJ_GRPO_K_FINALIZE = 3,
+  MJ_GRPO_K_DZ = 4,
+  MJ_GRPO_K_DHIDDEN = 5,
+  MJ_GRPO_K_DW = 6,
+  MJ_GRPO_K_REDUCE_LOSS = 7,
+  MJ_GRPO_K_COUNT = 8
+};
+int mj_grpo_profile_begin(int max_launches);
+int mj_grpo_profile_end(double* total_ms /* [MJ_GRPO_K_COUNT] */, int* launches /* [MJ_GRPO_K_COUNT] */);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MJ_GRPO_H */

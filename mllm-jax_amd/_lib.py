@@ -1,0 +1,88 @@
+"""ctypes binding of libmj_grpo.so (declarations: include/mj_grpo.h).
+
+There is no CPU fallback: if the library is missing or a call fails, this raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmj_grpo.so")
+
+OK = 0
+FLAG_DW_ACCUMULATE = 1 << 0
+FLAG_SFT = 1 << 1
+
+EXPORTS = ("mj_grpo_version", "mj_grpo_last_error", "mj_grpo_workspace_bytes", "mj_grpo_forward",
+           "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_profile_begin", "mj_grpo_profile_end")
+
+KERNEL_NAMES = ("k_transpose_bf16", "k_target_logit", "k_logits_stats", "k_finalize", "k_dz", "k_dhidden",
+                "k_dw", "k_reduce_loss")
+
+
+class MjGrpoDesc(C.Structure):
+    _fields_ = [
+        ("n_tokens", C.c_int64), ("hidden", C.c_int64), ("vocab", C.c_int64),
+        ("ld_hidden", C.c_int64), ("ld_w", C.c_int64), ("chunk_tokens", C.c_int64),
+        ("eps_low", C.c_float), ("eps_high", C.c_float), ("temperature", C.c_float),
+        ("softcap", C.c_float), ("inv_total_valid_tokens", C.c_float), ("grad_loss_scale", C.c_float),
+        ("flags", C.c_uint32), ("reserved", C.c_uint32),
+    ]
+
+
+class MjGrpoError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"mj_grpo status {code}: {message}")
+        self.code = code
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Loads the built library once; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f"{LIB_PATH} is missing: run `python -m mllm_jax_amd.build` (needs hipcc). "
+                           "There is no CPU fallback for the fused GRPO loss.")
+    lib = C.CDLL(LIB_PATH)
+    vp, fp, ip, sz = C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t
+    dp = C.POINTER(MjGrpoDesc)
+    lib.mj_grpo_version.restype = C.c_int
+    lib.mj_grpo_last_error.restype = C.c_char_p
+    lib.mj_grpo_workspace_bytes.argtypes = [dp, C.POINTER(sz), C.POINTER(sz)]
+    lib.mj_grpo_forward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp, sz, vp]
+    lib.mj_grpo_forward_backward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp, fp, vp, sz, vp]
+    lib.mj_grpo_backward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, vp, fp, vp, sz, vp]
+    lib.mj_grpo_profile_begin.argtypes = [C.c_int]
+    lib.mj_grpo_profile_end.argtypes = [C.POINTER(C.c_double), C.POINTER(C.c_int)]
+    for name in EXPORTS:
+        getattr(lib, name)
+    _lib = lib
+    return lib
+
+
+def check(status: int) -> None:
+    if status != OK:
+        raise MjGrpoError(status, load().mj_grpo_last_error().decode())
+
+
+def workspace_bytes(desc: MjGrpoDesc) -> tuple[int, int]:
+    f, b = C.c_size_t(0), C.c_size_t(0)
+    check(load().mj_grpo_workspace_bytes(C.byref(desc), C.byref(f), C.byref(b)))
+    return f.value, b.value
+
+
+def profile_begin(max_launches: int = 4096) -> None:
+    check(load().mj_grpo_profile_begin(max_launches))
+
+
+def profile_end() -> dict:
+    """{kernel name: (total_ms, launches)} since profile_begin."""
+    n = len(KERNEL_NAMES)
+    ms, cnt = (C.c_double * n)(), (C.c_int * n)()
+    check(load().mj_grpo_profile_end(ms, cnt))
+    return {KERNEL_NAMES[i]: (ms[i], cnt[i]) for i in range(n)}

@@ -1,0 +1,335 @@
+// mj_grpo.hip -- C ABI (include/mj_grpo.h) and launch plan of the fused GRPO loss path.
+#include "../../include/mj_grpo.h"
+
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "mj_grpo_kernels.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// ---- optional per-kernel timing with HIP events on the caller's stream (bench / profiling only)
+struct Profiler {
+  bool on = false;
+  hipEvent_t* ev = nullptr;
+  int* kid = nullptr;
+  int cap = 0, used = 0;   // event pairs
+} g_prof;
+
+struct Timed {
+  hipStream_t st;
+  bool active;
+  Timed(int kernel_id, hipStream_t s) : st(s), active(g_prof.on && g_prof.used < g_prof.cap) {
+    if (active) {
+      g_prof.kid[g_prof.used] = kernel_id;
+      (void)hipEventRecord(g_prof.ev[2 * g_prof.used], st);
+    }
+  }
+  ~Timed() {
+    if (active) {
+      (void)hipEventRecord(g_prof.ev[2 * g_prof.used + 1], st);
+      ++g_prof.used;
+    }
+  }
+};
+
+constexpr int BM = 256, BN = 256;          // tile of all three contractions
+constexpr int64_t kDefaultChunk = 8192;    // tokens whose logits live in the workspace at once
+
+inline int64_t rup(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
+
+struct Plan {
+  int64_t N, H, V, chunk, n_pad, parts, ld_ht;
+  // byte offsets into the workspace
+  size_t wt, zy, term, pm, pl, ps, g, ht, zt, dz, total_fwd, total_bwd;
+};
+
+int make_plan(const MjGrpoDesc* d, Plan* p) {
+  if (d == nullptr) return fail(MJ_GRPO_ERR_NULL, "desc is NULL");
+  if (d->n_tokens <= 0 || d->hidden <= 0 || d->vocab <= 0)
+    return fail(MJ_GRPO_ERR_SHAPE, "n_tokens/hidden/vocab must be positive (got %lld/%lld/%lld)",
+                (long long)d->n_tokens, (long long)d->hidden, (long long)d->vocab);
+  if (d->n_tokens > (1ll << 30) || d->hidden > (1 << 20) || d->vocab > (1 << 24))
+    return fail(MJ_GRPO_ERR_SHAPE, "shape too large");
+  if (d->ld_hidden < d->hidden || d->ld_w < d->vocab)
+    return fail(MJ_GRPO_ERR_SHAPE, "leading dimension smaller than row length");
+  if (d->hidden % 8 || d->vocab % 8 || d->ld_hidden % 8 || d->ld_w % 8)
+    return fail(MJ_GRPO_ERR_ALIGN, "hidden, vocab, ld_hidden and ld_w must be multiples of 8");
+  if (d->temperature != 1.0f)
+    return fail(MJ_GRPO_ERR_UNSUPPORTED, "temperature %g unsupported (only 1.0)", (double)d->temperature);
+  if (d->softcap < 0.f || !isfinite(d->softcap)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "softcap must be >= 0");
+  if (d->chunk_tokens < 0) return fail(MJ_GRPO_ERR_SHAPE, "chunk_tokens must be >= 0");
+  if (!isfinite(d->inv_total_valid_tokens)) return fail(MJ_GRPO_ERR_SHAPE, "inv_total_valid_tokens not finite");
+  p->N = d->n_tokens; p->H = d->hidden; p->V = d->vocab;
+  int64_t chunk = d->chunk_tokens > 0 ? d->chunk_tokens : kDefaultChunk;
+  chunk = rup(chunk, 256);
+  if (chunk > p->N) chunk = p->N;
+  p->chunk = chunk;
+  p->n_pad = rup(chunk, 256);
+  if (p->n_pad * p->V * 2 > (int64_t)0xffffffff)
+    return fail(MJ_GRPO_ERR_SHAPE, "chunk_tokens * vocab too large for one chunk; lower chunk_tokens");
+  p->parts = 2 * ((p->V + BM - 1) / BM);
+  p->ld_ht = rup(p->N, 64);
+  size_t o = 0;
+  auto take = [&](size_t bytes) { size_t at = o; o = (size_t)rup((int64_t)(o + bytes), 256); return at; };
+  p->wt = take((size_t)p->V * p->H * 2);
+  p->zy = take((size_t)p->N * 4);
+  p->term = take((size_t)p->N * 4);
+  p->pm = take((size_t)p->parts * p->n_pad * 4);
+  p->pl = take((size_t)p->parts * p->n_pad * 4);
+  p->ps = take((size_t)p->parts * p->n_pad * 4);
+  p->g = take((size_t)p->n_pad * 4);
+  p->total_fwd = o;
+  p->ht = take((size_t)p->H * p->ld_ht * 2);
+  p->zt = take((size_t)p->V * p->n_pad * 2);
+  p->dz = take((size_t)p->n_pad * p->V * 2);
+  p->total_bwd = o;
+  return MJ_GRPO_OK;
+}
+
+bool misaligned(const void* p) { return ((uintptr_t)p & 15u) != 0; }
+
+template <typename K>
+int enable_lds(K kernel) {
+  static thread_local const void* done[8] = {};
+  for (auto& d : done) if (d == (const void*)kernel) return MJ_GRPO_OK;
+  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     mj::GemmTN<BM, BN>::kLdsBytes);
+  if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  for (auto& d : done) if (d == nullptr) { d = (const void*)kernel; break; }
+  return MJ_GRPO_OK;
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  return MJ_GRPO_OK;
+}
+
+enum Mode { kForward, kForwardBackward, kBackwardOnly };
+
+int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head, const int32_t* targets,
+        const float* old_logp, const float* adv, const float* mask, float* logp, float* lse,
+        float* ent, float* loss, const float* saved_lse, const float* saved_logp, void* d_hidden,
+        float* d_w, void* workspace, size_t ws_bytes, void* stream_v) {
+  Plan p;
+  int rc = make_plan(d, &p);
+  if (rc) return rc;
+  const bool sft = (d->flags & MJ_GRPO_FLAG_SFT) != 0;
+  const bool bwd = mode != kForward;
+  if (!hidden || !lm_head || !targets || !mask) return fail(MJ_GRPO_ERR_NULL, "hidden/lm_head/targets/mask is NULL");
+  if (!sft && !adv) return fail(MJ_GRPO_ERR_NULL, "advantages is NULL");
+  if (mode != kBackwardOnly && (!logp || !lse || !loss)) return fail(MJ_GRPO_ERR_NULL, "logp/lse/loss output is NULL");
+  if (mode == kBackwardOnly && (!saved_lse || !saved_logp)) return fail(MJ_GRPO_ERR_NULL, "saved lse/logp is NULL");
+  if (bwd && (!d_hidden || !d_w)) return fail(MJ_GRPO_ERR_NULL, "d_hidden/d_lm_head is NULL");
+  if (!workspace) return fail(MJ_GRPO_ERR_WORKSPACE, "workspace is NULL");
+  const size_t need = bwd ? p.total_bwd : p.total_fwd;
+  if (ws_bytes < need) return fail(MJ_GRPO_ERR_WORKSPACE, "workspace too small: %zu < %zu bytes", ws_bytes, need);
+  if (misaligned(hidden) || misaligned(lm_head) || misaligned(workspace) || (bwd && misaligned(d_hidden)))
+    return fail(MJ_GRPO_ERR_ALIGN, "hidden, lm_head, d_hidden and workspace must be 16-byte aligned");
+
+  hipStream_t st = (hipStream_t)stream_v;
+  char* ws = (char*)workspace;
+  const int N = (int)p.N, H = (int)p.H, V = (int)p.V;
+  __bf16* wt = (__bf16*)(ws + p.wt);
+  float* zy = (float*)(ws + p.zy);
+  float* term = (float*)(ws + p.term);
+  float* pm = (float*)(ws + p.pm);
+  float* pl = (float*)(ws + p.pl);
+  float* ps = (float*)(ws + p.ps);
+  float* g = (float*)(ws + p.g);
+  __bf16* ht = (__bf16*)(ws + p.ht);
+  uint16_t* zt = (uint16_t*)(ws + p.zt);
+  uint16_t* dz = (uint16_t*)(ws + p.dz);
+  const float gscale = d->grad_loss_scale;
+  const size_t lds = mj::GemmTN<BM, BN>::kLdsBytes;
+
+  if ((rc = enable_lds(mj::k_logits_stats<BM, BN>))) return rc;
+  if (bwd) {
+    if ((rc = enable_lds(mj::k_dhidden<BM, BN>))) return rc;
+    if ((rc = enable_lds(mj::k_dw<BM, BN>))) return rc;
+  }
+
+  // lm_head[H,V] -> Wt[V,H]: K-contiguous operand of the logits product
+  {
+    Timed t(MJ_GRPO_K_TRANSPOSE, st);
+    mj::k_transpose_bf16<<<dim3((H + 63) / 64, (V + 63) / 64), 256, 0, st>>>(
+        (const uint16_t*)lm_head, d->ld_w, (uint16_t*)wt, H, H, V, H);
+  }
+  if (bwd) {   // hidden[N,H] -> hiddenT[H, ld_ht]: K-contiguous operand of the dW product
+    Timed t(MJ_GRPO_K_TRANSPOSE, st);
+    mj::k_transpose_bf16<<<dim3((unsigned)(p.ld_ht / 64), (H + 63) / 64), 256, 0, st>>>(
+        (const uint16_t*)hidden, d->ld_hidden, (uint16_t*)ht, p.ld_ht, N, H, (int)p.ld_ht);
+  }
+  if (mode != kBackwardOnly) {
+    Timed t(MJ_GRPO_K_TARGET_LOGIT, st);
+    mj::k_target_logit<<<(N + 3) / 4, 256, 0, st>>>((const __bf16*)hidden, d->ld_hidden, wt, H, targets, N,
+                                                    H, V, d->softcap, zy);
+  }
+  if ((rc = check_launch("prologue kernels"))) return rc;
+
+  for (int64_t c0 = 0; c0 < p.N; c0 += p.chunk) {
+    const int nc = (int)((p.N - c0 < p.chunk) ? p.N - c0 : p.chunk);
+    const int n_pad = (int)rup(nc, 256);
+    const __bf16* hid_c = (const __bf16*)hidden + c0 * d->ld_hidden;
+    {
+      mj::LogitsArgs a;
+      a.wt = wt; a.hid = hid_c; a.ld_wt = H; a.ld_hid = d->ld_hidden;
+      a.V = V; a.n = nc; a.H = H; a.cap = d->softcap;
+      a.zt = bwd ? zt : nullptr; a.ld_z = p.n_pad;
+      a.pm = pm; a.pl = pl; a.ps = ps; a.ld_p = p.n_pad;
+      mj::TileMap<4, 8> map((V + BM - 1) / BM, (nc + BN - 1) / BN);
+      Timed t(MJ_GRPO_K_LOGITS_STATS, st);
+      mj::k_logits_stats<BM, BN><<<map.grid(), mj::kThreads, lds, st>>>(a, map);
+    }
+    if (mode != kBackwardOnly) {
+      mj::FinalizeArgs f;
+      f.pm = pm; f.pl = pl; f.ps = ps; f.ld_p = p.n_pad; f.parts = (int)p.parts;
+      f.n = nc; f.n_pad = n_pad; f.zy = zy + c0;
+      f.old_logp = old_logp ? old_logp + c0 : nullptr;
+      f.adv = adv ? adv + c0 : nullptr; f.mask = mask + c0;
+      f.eps_low = d->eps_low; f.eps_high = d->eps_high; f.inv_tv = d->inv_total_valid_tokens;
+      f.gscale = gscale; f.sft = sft ? 1 : 0;
+      f.logp = logp + c0; f.lse = lse + c0; f.ent = ent ? ent + c0 : nullptr;
+      f.term = term + c0; f.g = bwd ? g : nullptr;
+      Timed t(MJ_GRPO_K_FINALIZE, st);
+      mj::k_finalize<<<n_pad / 64, 256, 0, st>>>(f);
+    } else {
+      Timed t(MJ_GRPO_K_FINALIZE, st);
+      mj::k_coeff_from_saved<<<(n_pad + 255) / 256, 256, 0, st>>>(
+          saved_logp + c0, old_logp ? old_logp + c0 : nullptr, adv ? adv + c0 : nullptr, mask + c0, nc, n_pad,
+          d->eps_low, d->eps_high, d->inv_total_valid_tokens, gscale, sft ? 1 : 0, g);
+    }
+    if (bwd) {
+      mj::DzArgs z;
+      z.zt = zt; z.ld_z = p.n_pad; z.dz = dz; z.ld_dz = V;
+      z.lse = (mode == kBackwardOnly ? saved_lse : lse) + c0; z.g = g; z.targets = targets + c0;
+      z.V = V; z.n = nc; z.n_pad = n_pad; z.cap = d->softcap;
+      {
+        Timed t(MJ_GRPO_K_DZ, st);
+        mj::k_dz<<<dim3((V + 63) / 64, n_pad / 64), 256, 0, st>>>(z);
+      }
+
+      mj::DhArgs h;
+      h.dz = (const __bf16*)dz; h.w = (const __bf16*)lm_head; h.ld_dz = V; h.ld_w = d->ld_w;
+      h.n = nc; h.H = H; h.V = V;
+      h.dh = (uint16_t*)d_hidden + c0 * d->ld_hidden; h.ld_dh = d->ld_hidden;
+      mj::TileMap<4, 8> mh((nc + BM - 1) / BM, (H + BN - 1) / BN);
+      {
+        Timed t(MJ_GRPO_K_DHIDDEN, st);
+        mj::k_dhidden<BM, BN><<<mh.grid(), mj::kThreads, lds, st>>>(h, mh);
+      }
+
+      mj::DwArgs w;
+      w.ht = ht + c0; w.dzt = (const __bf16*)zt; w.ld_ht = p.ld_ht; w.ld_z = p.n_pad;
+      w.H = H; w.V = V; w.K = (int)rup(nc, 8);
+      w.dw = d_w; w.ld_dw = d->ld_w;
+      w.accumulate = (c0 > 0 || (d->flags & MJ_GRPO_FLAG_DW_ACCUMULATE)) ? 1 : 0;
+      mj::TileMap<4, 8> mw((H + BM - 1) / BM, (V + BN - 1) / BN);
+      {
+        Timed t(MJ_GRPO_K_DW, st);
+        mj::k_dw<BM, BN><<<mw.grid(), mj::kThreads, lds, st>>>(w, mw);
+      }
+    }
+    if ((rc = check_launch("chunk kernels"))) return rc;
+  }
+  if (mode != kBackwardOnly) {
+    {
+      Timed t(MJ_GRPO_K_REDUCE_LOSS, st);
+      mj::k_reduce_loss<<<1, 1024, 0, st>>>(term, N, loss);
+    }
+    if ((rc = check_launch("k_reduce_loss"))) return rc;
+  }
+  return MJ_GRPO_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mj_grpo_version(void) { return 100; }
+
+const char* mj_grpo_last_error(void) { return g_err; }
+
+int mj_grpo_profile_begin(int max_launches) {
+  if (g_prof.on) return fail(MJ_GRPO_ERR_UNSUPPORTED, "profiling already on");
+  if (max_launches <= 0 || max_launches > (1 << 16)) return fail(MJ_GRPO_ERR_SHAPE, "max_launches out of range");
+  g_prof.ev = new hipEvent_t[2 * (size_t)max_launches];
+  g_prof.kid = new int[max_launches];
+  for (int i = 0; i < 2 * max_launches; ++i) {
+    hipError_t e = hipEventCreate(&g_prof.ev[i]);
+    if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipEventCreate: %s", hipGetErrorString(e));
+  }
+  g_prof.cap = max_launches;
+  g_prof.used = 0;
+  g_prof.on = true;
+  return MJ_GRPO_OK;
+}
+
+int mj_grpo_profile_end(double* total_ms, int* launches) {
+  if (!g_prof.on) return fail(MJ_GRPO_ERR_UNSUPPORTED, "profiling is not on");
+  if (!total_ms || !launches) return fail(MJ_GRPO_ERR_NULL, "total_ms/launches is NULL");
+  for (int k = 0; k < MJ_GRPO_K_COUNT; ++k) { total_ms[k] = 0.0; launches[k] = 0; }
+  int rc = MJ_GRPO_OK;
+  for (int i = 0; i < g_prof.used; ++i) {
+    float ms = 0.f;
+    hipError_t e = hipEventSynchronize(g_prof.ev[2 * i + 1]);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, g_prof.ev[2 * i], g_prof.ev[2 * i + 1]);
+    if (e != hipSuccess) { rc = fail(MJ_GRPO_ERR_HIP, "profile event: %s", hipGetErrorString(e)); break; }
+    total_ms[g_prof.kid[i]] += ms;
+    launches[g_prof.kid[i]] += 1;
+  }
+  for (int i = 0; i < 2 * g_prof.cap; ++i) (void)hipEventDestroy(g_prof.ev[i]);
+  delete[] g_prof.ev;
+  delete[] g_prof.kid;
+  g_prof = Profiler();
+  return rc;
+}
+
+int mj_grpo_workspace_bytes(const MjGrpoDesc* desc, size_t* forward_bytes, size_t* forward_backward_bytes) {
+  Plan p;
+  int rc = make_plan(desc, &p);
+  if (rc) return rc;
+  if (forward_bytes) *forward_bytes = p.total_fwd;
+  if (forward_backward_bytes) *forward_backward_bytes = p.total_bwd;
+  return MJ_GRPO_OK;
+}
+
+int mj_grpo_forward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head, const int32_t* targets,
+                    const float* old_logp, const float* advantages, const float* mask, float* logp,
+                    float* lse, float* token_entropy, float* loss, void* workspace, size_t workspace_bytes,
+                    void* stream) {
+  return run(kForward, desc, hidden, lm_head, targets, old_logp, advantages, mask, logp, lse, token_entropy,
+             loss, nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, stream);
+}
+
+int mj_grpo_forward_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
+                             const int32_t* targets, const float* old_logp, const float* advantages,
+                             const float* mask, float* logp, float* lse, float* token_entropy, float* loss,
+                             void* d_hidden, float* d_lm_head, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+  return run(kForwardBackward, desc, hidden, lm_head, targets, old_logp, advantages, mask, logp, lse,
+             token_entropy, loss, nullptr, nullptr, d_hidden, d_lm_head, workspace, workspace_bytes, stream);
+}
+
+int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head, const int32_t* targets,
+                     const float* old_logp, const float* advantages, const float* mask, const float* lse,
+                     const float* logp, void* d_hidden, float* d_lm_head, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+  return run(kBackwardOnly, desc, hidden, lm_head, targets, old_logp, advantages, mask, nullptr, nullptr,
+             nullptr, nullptr, lse, logp, d_hidden, d_lm_head, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,289 @@
+"""Host side of the fused GRPO loss: the reference's loss-function contract on top of
+the HIP kernels in libmj_grpo.so.
+
+Mirrors, for the lm_head + loss part only:
+  MLLM_JAX/train_modules/__init__.py:84-192   TrainGRPOModule (inputs / outputs, hyper-parameters)
+  plugins/training/update/train_step.py:15-24 loss_fn + jax.value_and_grad(has_aux=True)
+  plugins/sft/jax/sft_module.py:22-45         TrainSftModule (masked cross-entropy)
+
+torch is used for device memory, streams and autograd plumbing only; all arithmetic on
+[tokens, vocab]-sized data happens in the HIP kernels.  No CPU fallback exists.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Any, Callable, Mapping, Optional
+
+import torch
+
+from . import _lib
+
+_workspaces: dict[Any, torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    key = (device.type, device.index)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        _workspaces.pop(key, None)
+        ws = None
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def release_workspaces() -> None:
+    """Drops the cached per-device workspaces."""
+    _workspaces.clear()
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _as_f32(x, n: int, device, name: str) -> torch.Tensor:
+    t = torch.as_tensor(x, device=device)
+    if t.numel() != n:
+        raise ValueError(f"{name} has {t.numel()} elements, expected {n}")
+    return t.reshape(n).to(torch.float32).contiguous()
+
+
+class _Prepared:
+    """Validated, flattened device arguments of one call."""
+
+    def __init__(self, hidden, lm_head, target_ids, old_logps, advantages, mask, *,
+                 total_valid_token_count, epsilon_low, epsilon_high, temperature,
+                 final_logit_softcap, seq_shape, chunk_tokens, sft=False, accumulate=False):
+        if hidden.device.type != "cuda":
+            raise RuntimeError("grpo_fused_loss needs tensors on an MI355X device (got "
+                               f"{hidden.device}); there is no CPU path")
+        if hidden.dim() == 3:
+            if seq_shape is None:
+                seq_shape = (hidden.shape[0], hidden.shape[1])
+            hidden = hidden.reshape(-1, hidden.shape[-1])
+        if hidden.dim() != 2 or lm_head.dim() != 2 or hidden.shape[1] != lm_head.shape[0]:
+            raise ValueError(f"hidden {tuple(hidden.shape)} and lm_head {tuple(lm_head.shape)} do not "
+                             "form [N,H] x [H,V]")
+        n, h = hidden.shape
+        v = lm_head.shape[1]
+        if seq_shape is not None and seq_shape[0] * seq_shape[1] != n:
+            raise ValueError(f"seq_shape {seq_shape} does not match {n} tokens")
+        dev = hidden.device
+        self.n, self.h, self.v, self.seq_shape, self.device = n, h, v, seq_shape, dev
+        self.hidden = hidden.to(torch.bfloat16)
+        if self.hidden.stride(1) != 1 or self.hidden.stride(0) % 8:
+            self.hidden = self.hidden.contiguous()
+        self.w = lm_head.detach().to(torch.bfloat16)
+        if self.w.stride(1) != 1 or self.w.stride(0) % 8:
+            self.w = self.w.contiguous()
+        self.targets = torch.as_tensor(target_ids, device=dev).reshape(-1).to(torch.int32).contiguous()
+        if self.targets.numel() != n:
+            raise ValueError(f"target_ids has {self.targets.numel()} elements, expected {n}")
+        self.mask = _as_f32(mask, n, dev, "mask")
+        self.old = None if old_logps is None else _as_f32(old_logps, n, dev, "old_logps")
+        if sft:
+            self.adv = None
+        else:
+            adv = torch.as_tensor(advantages, device=dev).to(torch.float32)
+            if adv.numel() != n:
+                # the reference passes [B] and broadcasts over the sequence (train_modules/__init__.py:173)
+                if seq_shape is None or adv.numel() != seq_shape[0]:
+                    raise ValueError(f"advantages has {adv.numel()} elements; expected {n} tokens or "
+                                     "one per sequence with seq_shape given")
+                adv = adv.reshape(-1, 1).expand(seq_shape[0], seq_shape[1])
+            self.adv = adv.reshape(n).contiguous()
+        if total_valid_token_count is None:
+            tv = float(self.mask.sum().item())       # reference default: mask.sum() (:179)
+            if sft:
+                tv = max(tv, 1.0)                    # sft_module.py:14
+        else:
+            tv = float(total_valid_token_count)
+        self.tv = tv
+        d = _lib.MjGrpoDesc()
+        d.n_tokens, d.hidden, d.vocab = n, h, v
+        d.ld_hidden, d.ld_w = self.hidden.stride(0), self.w.stride(0)
+        d.chunk_tokens = int(chunk_tokens or 0)
+        d.eps_low, d.eps_high = float(epsilon_low), float(epsilon_high)
+        d.temperature = float(temperature)
+        d.softcap = float(final_logit_softcap or 0.0)
+        d.inv_total_valid_tokens = (1.0 / tv) if tv != 0 else float("inf")
+        d.grad_loss_scale = 1.0
+        d.flags = (_lib.FLAG_SFT if sft else 0) | (_lib.FLAG_DW_ACCUMULATE if accumulate else 0)
+        self.desc = d
+        self.logp = torch.empty(n, dtype=torch.float32, device=dev)
+        self.lse = torch.empty(n, dtype=torch.float32, device=dev)
+        self.ent = torch.empty(n, dtype=torch.float32, device=dev)
+        self.loss = torch.empty(1, dtype=torch.float32, device=dev)
+
+    def stream(self) -> int:
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def forward(self) -> None:
+        fwd, _ = _lib.workspace_bytes(self.desc)
+        ws = _workspace(self.device, fwd)
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.load().mj_grpo_forward(
+                C.byref(self.desc), _ptr(self.hidden), _ptr(self.w), _ptr(self.targets), _ptr(self.old),
+                _ptr(self.adv), _ptr(self.mask), _ptr(self.logp), _ptr(self.lse), _ptr(self.ent),
+                _ptr(self.loss), _ptr(ws), ws.numel(), self.stream()))
+
+    def forward_backward(self, d_w: Optional[torch.Tensor] = None):
+        _, both = _lib.workspace_bytes(self.desc)
+        ws = _workspace(self.device, both)
+        d_h = torch.empty_like(self.hidden)
+        if d_w is None:
+            d_w = torch.empty((self.h, self.w.stride(0)), dtype=torch.float32, device=self.device)
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.load().mj_grpo_forward_backward(
+                C.byref(self.desc), _ptr(self.hidden), _ptr(self.w), _ptr(self.targets), _ptr(self.old),
+                _ptr(self.adv), _ptr(self.mask), _ptr(self.logp), _ptr(self.lse), _ptr(self.ent),
+                _ptr(self.loss), _ptr(d_h), _ptr(d_w), _ptr(ws), ws.numel(), self.stream()))
+        return d_h, d_w[:, : self.v]
+
+    def metrics(self, return_token_entropy: bool, sft: bool = False) -> dict:
+        """The reference's return dict (train_modules/__init__.py:185-192)."""
+        out = {"loss": self.loss[0]}
+        shape = self.seq_shape if self.seq_shape is not None else (self.n,)
+        out["per_token_logps"] = self.logp.reshape(shape)
+        if sft:
+            out["token_count"] = self.mask.sum().to(torch.int32)
+            return out
+        if self.seq_shape is not None:
+            b, t = self.seq_shape
+            ent = self.ent.reshape(b, t)
+            m = self.mask.reshape(b, t)
+            out["entropy"] = (ent * m).sum(-1) / m.sum(-1)                    # :141-143
+            valid = m == 1
+            cum = torch.cumsum(valid, dim=-1)
+            win = (valid & (cum >= 4) & (cum <= 100)).to(torch.float32)      # :148-153
+            out["entropy_loss"] = (ent * win).sum(-1) / win.sum(-1)          # :155-157
+        if return_token_entropy:
+            out["token_entropy"] = self.ent.reshape(shape)
+        return out
+
+
+_DEFAULTS = dict(total_valid_token_count=None, epsilon_low=0.2, epsilon_high=0.3, temperature=1.0,
+                 final_logit_softcap=None, seq_shape=None, chunk_tokens=None)
+
+
+def grpo_loss_value_and_grad(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
+                             return_token_entropy=False, accumulate_into=None, **kw):
+    """value_and_grad form of the loss, the call shape of the reference's train step
+    (plugins/training/update/train_step.py:24): returns (metrics, (d_hidden, d_lm_head)).
+
+    d_hidden is bf16 [N,H]; d_lm_head is float32 [H,V] (the reference's parameter gradients
+    are float32).  `accumulate_into` (a float32 [H,V] tensor) makes the kernel add into an
+    existing gradient buffer instead of overwriting (grad accumulation, train_step.py:30-33).
+    One fused pass: 6*N*H*V flop, 16-bit logits of at most `chunk_tokens` tokens in the workspace."""
+    opts = {**_DEFAULTS, **kw}
+    p = _Prepared(hidden, lm_head, target_ids, old_logps, advantages, mask,
+                  accumulate=accumulate_into is not None, **opts)
+    if accumulate_into is not None:
+        if accumulate_into.dtype != torch.float32 or tuple(accumulate_into.shape) != (p.h, p.v) \
+                or accumulate_into.stride(1) != 1 or accumulate_into.stride(0) != p.w.stride(0):
+            raise ValueError("accumulate_into must be a float32 [H,V] tensor laid out like lm_head")
+    d_h, d_w = p.forward_backward(accumulate_into)
+    return p.metrics(return_token_entropy), (d_h.reshape(hidden.shape), d_w)
+
+
+class _FusedLossFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, hidden, lm_head, prepared: _Prepared, want_grad: bool):
+        if want_grad:
+            d_h, d_w = prepared.forward_backward()
+            ctx.save_for_backward(d_h, d_w)
+            ctx.shapes = (hidden.shape, hidden.dtype, lm_head.dtype)
+        else:
+            prepared.forward()
+        return prepared.loss[0].clone()
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        d_h, d_w = ctx.saved_tensors
+        shape, h_dtype, w_dtype = ctx.shapes
+        gh = (d_h * grad_loss.to(d_h.dtype)).reshape(shape).to(h_dtype)
+        gw = (d_w * grad_loss).to(w_dtype)
+        return gh, gw, None, None
+
+
+def grpo_fused_loss(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
+                    return_token_entropy=False, **kw) -> dict:
+    """The reference's loss contract on flattened tokens.
+
+    hidden [N,H] or [B,T,H] bf16, lm_head [H,V] bf16 (or float32 master weights),
+    target_ids [N] int, old_logps [N] float32 or None (None = on-policy, ratio 1,
+    train_modules/__init__.py:161-165), advantages [N] (or [B] with seq_shape=(B,T)),
+    mask [N] in {0,1}.  Returns {"loss", "per_token_logps", "entropy", "entropy_loss"
+    [, "token_entropy"]} like train_modules/__init__.py:185-192; "loss" is differentiable
+    with respect to hidden and lm_head, everything else carries no gradient."""
+    opts = {**_DEFAULTS, **kw}
+    p = _Prepared(hidden, lm_head, target_ids, old_logps, advantages, mask, **opts)
+    want = torch.is_grad_enabled() and (hidden.requires_grad or lm_head.requires_grad)
+    loss = _FusedLossFn.apply(hidden, lm_head, p, want)
+    out = p.metrics(return_token_entropy)
+    out["loss"] = loss
+    return out
+
+
+def sft_fused_loss(hidden, lm_head, labels, valid, **kw) -> dict:
+    """Masked next-token cross-entropy of plugins/sft/jax/sft_module.py:22-45 on already
+    shifted, flattened tokens: loss = sum(-logp * valid) / max(sum(valid), 1).  Positions with
+    valid == 0 may hold any label (the reference maps them to 0, :35)."""
+    opts = {**_DEFAULTS, **kw}
+    labels = torch.as_tensor(labels, device=hidden.device)
+    validb = torch.as_tensor(valid, device=hidden.device).reshape(-1).bool()
+    safe = torch.where(validb, labels.reshape(-1), torch.zeros_like(labels.reshape(-1)))
+    p = _Prepared(hidden, lm_head, safe, None, None, validb.to(torch.float32), sft=True, **opts)
+    want = torch.is_grad_enabled() and (hidden.requires_grad or lm_head.requires_grad)
+    loss = _FusedLossFn.apply(hidden, lm_head, p, want)
+    out = p.metrics(False, sft=True)
+    out["loss"] = loss
+    return out
+
+
+class TrainGRPOModule:
+    """Drop-in for the reference's TrainGRPOModule (MLLM_JAX/train_modules/__init__.py:84-192)
+    with the lm_head product fused into the loss.
+
+    `model(input_ids=..., attention_mask=...)` returns the FINAL HIDDEN STATES [B,L,H] (what
+    Qwen2Model returns before lm_head, qwen2/modular_qwen2.py:161) and `lm_head` is the
+    [H,V] kernel (or a zero-argument callable returning it).  `__call__(inputs)` takes the
+    reference's batch dict (input_ids, attention_mask, labels, advantages and optionally
+    old_per_token_logps, total_valid_token_count) and returns its metrics dict."""
+
+    def __init__(self, model: Callable, lm_head, pad_token_id: float = 0, num_pre_Q: int = 1,
+                 ref_model: Any = None, beta: float = 0.04, temperature: float = 1.0,
+                 max_lengths: float = 2048, epsilon_low: float = 0.2, epsilon_high: float = 0.3,
+                 entropy_threshold: float = 0.3, final_logit_softcap: Optional[float] = None,
+                 chunk_tokens: Optional[int] = None):
+        self.model, self.lm_head = model, lm_head
+        self.pad_token_id, self.num_pre_Q, self.ref_model, self.beta = pad_token_id, num_pre_Q, ref_model, beta
+        self.temperature, self.max_lengths = temperature, max_lengths
+        self.epsilon_low, self.epsilon_high = epsilon_low, epsilon_high
+        self.entropy_threshold = entropy_threshold
+        self.final_logit_softcap, self.chunk_tokens = final_logit_softcap, chunk_tokens
+
+    def __call__(self, inputs: Mapping[str, Any]) -> dict:
+        input_ids, labels = inputs["input_ids"], inputs["labels"]
+        hidden = self.model(input_ids=input_ids, attention_mask=inputs["attention_mask"])
+        w = self.lm_head() if callable(self.lm_head) else self.lm_head
+        b, l = input_ids.shape
+        hid = hidden[:, :-1, :]                       # logits[..., :-1, :]   (:124)
+        chosen = input_ids[:, 1:]                     # :118
+        mask = labels[:, 1:]                          # :120
+        return grpo_fused_loss(
+            hid.reshape(b * (l - 1), -1), w, chosen.reshape(-1), inputs.get("old_per_token_logps"),
+            inputs["advantages"], mask.reshape(-1),
+            total_valid_token_count=inputs.get("total_valid_token_count"),
+            epsilon_low=self.epsilon_low, epsilon_high=self.epsilon_high, temperature=self.temperature,
+            final_logit_softcap=self.final_logit_softcap, seq_shape=(b, l - 1),
+            chunk_tokens=self.chunk_tokens)
+
+
+def loss_and_metrics(module: Callable[[Mapping[str, Any]], dict], inputs: Mapping[str, Any]):
+    """loss_fn of plugins/training/update/train_step.py:15-22: pops per_token_logps, means
+    the other metrics, returns (loss, metrics | {"per_token_logps": ...})."""
+    metrics = dict(module(inputs))
+    per_token_logps = metrics.pop("per_token_logps", None)
+    metrics = {k: torch.mean(v.float()) for k, v in metrics.items()}
+    return metrics["loss"], {**metrics, "per_token_logps": per_token_logps}

@@ -186,32 +186,35 @@ def sft_cross_entropy(hidden, lm_head, labels, valid, *, with_grads=True):
 def grpo_loss_chunked_torch(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
                             total_valid_token_count=None, epsilon_low=0.2, epsilon_high=0.3,
                             final_logit_softcap=None, with_grads=True, chunk=1024,
-                            dtype=None, rows=None):
-    """Same arithmetic as grpo_loss (temperature 1) in torch on the CPU, token-chunked
-    so BASELINE-sized shapes fit in host memory.  float32 matmul by default (inputs are
-    bf16-valued, so products are exact and only the accumulation rounds), float64
-    softmax statistics.  `rows` restricts the work to a subset of token rows while the
-    normaliser stays that of the whole batch; d_lm_head is then that subset's share."""
+                            dtype=None, rows=None, device="cpu", as_numpy=True):
+    """Same arithmetic as grpo_loss (temperature 1) in torch, token-chunked so that
+    BASELINE-sized shapes fit in memory.  float32 matmul by default (inputs are bf16-valued,
+    so products are exact and only the accumulation rounds), float64 softmax statistics.
+    `device` may name the GPU for the full-size configurations: the matmuls are then
+    torch's own float32 GEMMs, still independent of the kernels under test.  `rows`
+    restricts the work to a subset of token rows while the normaliser stays that of the
+    whole batch; d_lm_head is then that subset's share."""
     import torch
 
     dt = dtype or torch.float32
-    h = torch.as_tensor(hidden).to(dt)
-    w = torch.as_tensor(lm_head).to(dt)
-    y = torch.as_tensor(target_ids).long()
-    adv = torch.as_tensor(advantages).double()
-    m = torch.as_tensor(mask).double()
+    dev = torch.device(device)
+    h = torch.as_tensor(hidden).to(dev).to(dt)
+    w = torch.as_tensor(lm_head).to(dev).to(dt)
+    y = torch.as_tensor(target_ids).to(dev).long()
+    adv = torch.as_tensor(advantages).to(dev).double()
+    m = torch.as_tensor(mask).to(dev).double()
     n = h.shape[0]
     tv = float(m.sum()) if total_valid_token_count is None else float(total_valid_token_count)
-    old = None if old_logps is None else torch.as_tensor(old_logps).double()
-    idx = torch.arange(n) if rows is None else torch.as_tensor(rows).long()
+    old = None if old_logps is None else torch.as_tensor(old_logps).to(dev).double()
+    idx = torch.arange(n, device=dev) if rows is None else torch.as_tensor(rows).to(dev).long()
     cap = float(final_logit_softcap) if final_logit_softcap else None
     lo, hi = 1.0 - float(epsilon_low), 1.0 + float(epsilon_high)
-    logp = torch.zeros(n, dtype=torch.float64)
-    lse = torch.zeros(n, dtype=torch.float64)
-    ent = torch.zeros(n, dtype=torch.float64)
-    ptl = torch.zeros(n, dtype=torch.float64)
-    d_h = torch.zeros(h.shape, dtype=torch.float32) if with_grads else None
-    d_w = torch.zeros(w.shape, dtype=torch.float32) if with_grads else None
+    logp = torch.zeros(n, dtype=torch.float64, device=dev)
+    lse = torch.zeros(n, dtype=torch.float64, device=dev)
+    ent = torch.zeros(n, dtype=torch.float64, device=dev)
+    ptl = torch.zeros(n, dtype=torch.float64, device=dev)
+    d_h = torch.zeros(h.shape, dtype=torch.float32, device=dev) if with_grads else None
+    d_w = torch.zeros(w.shape, dtype=torch.float32, device=dev) if with_grads else None
     for s in range(0, idx.numel(), chunk):
         r = idx[s:s + chunk]
         z = (h[r] @ w).double()
@@ -232,17 +235,19 @@ def grpo_loss_chunked_torch(hidden, lm_head, target_ids, old_logps, advantages, 
             active = ((ratio >= lo) & (ratio <= hi)) | ((ratio > hi) & (a < 0)) | ((ratio < lo) & (a > 0))
             g = -(m[r] / tv) * a * ratio * active
             dz = -p
-            dz.scatter_add_(1, y[r, None], torch.ones(len(r), 1, dtype=torch.float64))
+            dz.scatter_add_(1, y[r, None], torch.ones(len(r), 1, dtype=torch.float64, device=dev))
             dz *= g[:, None]
             if cap:
                 dz *= 1.0 - (z / cap) ** 2
             dzf = dz.to(dt)
             d_h[r] = (dzf @ w.T).float()
             d_w += (h[r].T @ dzf).float()
+            del dz, dzf
+        del z, p
     loss = float((ptl * m).sum() / tv)
-    out = {"loss": loss, "per_token_logps": logp.numpy(), "lse": lse.numpy(),
-           "token_entropy": ent.numpy()}
+    conv = (lambda t: t.cpu().numpy()) if as_numpy else (lambda t: t)
+    out = {"loss": loss, "per_token_logps": conv(logp), "lse": conv(lse), "token_entropy": conv(ent)}
     if with_grads:
-        out["d_hidden"] = d_h.numpy()
-        out["d_lm_head"] = d_w.numpy()
+        out["d_hidden"] = conv(d_h)
+        out["d_lm_head"] = conv(d_w)
     return out

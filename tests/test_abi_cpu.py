@@ -1,0 +1,110 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol that
+include/mj_grpo.h declares, and rejects bad descriptors / pointers with a status and a
+message before touching any device (no compute call is made here)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from mllm_jax_amd import _lib, build
+    if not os.path.exists(_lib.LIB_PATH):
+        build.build(verbose=False)
+    return _lib
+
+
+def _desc(lib, **kw):
+    d = lib.MjGrpoDesc()
+    d.n_tokens, d.hidden, d.vocab, d.ld_hidden, d.ld_w = 64, 64, 512, 64, 512
+    d.temperature, d.inv_total_valid_tokens, d.grad_loss_scale = 1.0, 1.0 / 64, 1.0
+    d.eps_low, d.eps_high = 0.2, 0.3
+    for k, v in kw.items():
+        setattr(d, k, v)
+    return d
+
+
+def test_header_symbols_are_exported(lib):
+    header = open(os.path.join(ROOT, "include", "mj_grpo.h")).read()
+    declared = set(re.findall(r"\b(mj_grpo_[a-z_]+)\s*\(", header))
+    assert declared == set(lib.EXPORTS)
+    handle = lib.load()
+    for name in declared:
+        assert hasattr(handle, name)
+    assert handle.mj_grpo_version() >= 100
+
+
+def test_desc_layout_matches_header(lib):
+    # 6 x int64 + 6 x float + 2 x uint32
+    assert C.sizeof(lib.MjGrpoDesc) == 6 * 8 + 6 * 4 + 2 * 4
+
+
+def test_workspace_sizes_scale_with_chunk(lib):
+    big = _desc(lib, n_tokens=16384, hidden=3584, vocab=152064, ld_hidden=3584, ld_w=152064)
+    f, b = lib.workspace_bytes(big)
+    small = _desc(lib, n_tokens=16384, hidden=3584, vocab=152064, ld_hidden=3584, ld_w=152064, chunk_tokens=2048)
+    f2, b2 = lib.workspace_bytes(small)
+    assert f2 < f and b2 < b
+    # the workspace never holds N x V logits: two 16-bit chunk buffers + transposed operands
+    assert b2 < 16384 * 152064 * 2
+
+
+@pytest.mark.parametrize("kw,code", [
+    (dict(n_tokens=0), 2), (dict(vocab=-8), 2), (dict(ld_w=256), 2),
+    (dict(vocab=508, ld_w=508), 3), (dict(hidden=60, ld_hidden=60), 3), (dict(ld_hidden=68), 3),
+    (dict(temperature=0.7), 5), (dict(softcap=-1.0), 5), (dict(chunk_tokens=-5), 2),
+    (dict(inv_total_valid_tokens=float("inf")), 2),
+])
+def test_bad_descriptors(lib, kw, code):
+    with pytest.raises(lib.MjGrpoError) as e:
+        lib.workspace_bytes(_desc(lib, **kw))
+    assert e.value.code == code and len(str(e.value)) > 20
+
+
+def test_null_and_workspace_errors_before_any_launch(lib):
+    h = lib.load()
+    d = _desc(lib)
+    fake = 0x1000   # never dereferenced: argument checks fail first
+    st = h.mj_grpo_forward(C.byref(d), None, fake, fake, None, fake, fake, fake, fake, None, fake, fake, 1 << 30, None)
+    assert st == 1 and b"NULL" in h.mj_grpo_last_error()
+    st = h.mj_grpo_forward(C.byref(d), fake, fake, fake, None, fake, fake, fake, fake, None, fake, None, 0, None)
+    assert st == 4
+    st = h.mj_grpo_forward(C.byref(d), fake, fake, fake, None, fake, fake, fake, fake, None, fake, fake, 16, None)
+    assert st == 4 and b"too small" in h.mj_grpo_last_error()
+    st = h.mj_grpo_forward(C.byref(d), fake + 2, fake, fake, None, fake, fake, fake, fake, None, fake, fake, 1 << 30, None)
+    assert st == 3
+    st = h.mj_grpo_forward_backward(C.byref(d), fake, fake, fake, None, fake, fake, fake, fake, None, fake, None,
+                                    fake, fake, 1 << 30, None)
+    assert st == 1
+    st = h.mj_grpo_backward(C.byref(d), fake, fake, fake, None, fake, fake, None, fake, fake, fake, fake, 1 << 30, None)
+    assert st == 1
+    st = h.mj_grpo_forward(None, fake, fake, fake, None, fake, fake, fake, fake, None, fake, fake, 1 << 30, None)
+    assert st == 1
+
+
+def test_host_api_refuses_cpu_tensors(lib):
+    import torch
+    import mllm_jax_amd as M
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        M.grpo_fused_loss(torch.zeros(8, 8, dtype=torch.bfloat16), torch.zeros(8, 16, dtype=torch.bfloat16),
+                          torch.zeros(8, dtype=torch.long), None, torch.zeros(8), torch.ones(8))
+
+
+def test_workload_generator_shapes_and_advantages():
+    import numpy as np
+    import torch
+    from mllm_jax_amd import CONFIGS, make_workload
+    from mllm_jax_amd.workloads import group_advantages
+    from oracle.grpo_oracle import grpo_advantages
+    r = torch.tensor([1.0, 0, 0, 1, 1, 1, 0, 0])
+    np.testing.assert_allclose(group_advantages(r, 4).numpy(), grpo_advantages(r.numpy(), [0] * 4 + [1] * 4), rtol=1e-6)
+    assert [c.tokens for c in CONFIGS] == [512, 4096, 16384, 32768, 16384]
+    import dataclasses
+    tiny = dataclasses.replace(CONFIGS[0], hidden=16, vocab=64)
+    wl = make_workload(tiny, "cpu", 1)
+    assert wl["hidden"].shape == (512, 16) and wl["lm_head"].shape == (16, 64)
+    assert wl["advantages"].abs().max() > 0 and wl["total_valid_token_count"] == wl["mask"].sum().item()
