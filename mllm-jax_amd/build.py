@@ -39,6 +39,8 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+    import ctypes
+    ctypes.CDLL(LIB + ".tmp")          # an unresolved symbol must fail the build, not the first call
     os.replace(LIB + ".tmp", LIB)
     return LIB
 

@@ -333,3 +333,8 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
 }
 
 }  // extern "C"
+
+// Explicit instantiations of the tile kernels used above.
+template __global__ void mj::k_logits_stats<256, 256>(mj::LogitsArgs, mj::TileMap<4, 8>);
+template __global__ void mj::k_dhidden<256, 256>(mj::DhArgs, mj::TileMap<4, 8>);
+template __global__ void mj::k_dw<256, 256>(mj::DwArgs, mj::TileMap<4, 8>);
