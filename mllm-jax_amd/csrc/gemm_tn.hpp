@@ -4,13 +4,16 @@
 // One workgroup of 256 threads (4 wavefronts, 2x2) owns a BM x BN tile; each wavefront owns
 // (BM/2) x (BN/2) as a grid of 32x32 MFMA blocks (v_mfma_f32_32x32x16_bf16).
 //
-// K is walked in slices of 32 through a ring of LDS stages.  Global memory is copied straight
-// into LDS (buffer_load_dwordx4 ... lds: no staging registers, no ds_write), several slices
-// ahead of the MFMAs, so the load latency is covered by (STAGES-1) slices of math.  Rows past the
-// operand's end read as zero through the buffer descriptor's range check; K tails are masked
-// per 16-byte chunk.  The LDS image of a slice is 64 bytes per row; the 16-byte chunk a lane
-// fetches is XOR-permuted within its row so that the ds_read_b128 of 16 consecutive rows hits 16
-// different bank groups.
+// K is walked in slices of 64 through two LDS stages.  A slice travels global memory ->
+// registers (16-byte buffer loads, every 8 lanes cover one full 128-byte line of a tile row) ->
+// LDS (ds_write_b128) -> MFMA operands (ds_read_b128).  The loads of slice k+2 and the LDS writes
+// of slice k+1 are issued one at a time between the MFMAs of slice k, so the texture-address unit
+// sees an even trickle instead of a burst and every load has a whole slice of math to land.  Rows
+// past the operand's end read as zero through the buffer descriptor's range check; K tails are
+// masked per 16-byte chunk.  The LDS image of a slice is 128 bytes per row; 16-byte chunk c of
+// row r sits at slot c ^ swz(r), which keeps both the writes and the ds_read_b128 of consecutive
+// rows bank-conflict free whether the LDS serves 8 or 16 lanes per clock.  MFMA operands are
+// double-buffered in registers: the LDS reads of k-step s+1 sit between the MFMAs of k-step s.
 //
 // The three contractions of the loss path are instances of this engine with different epilogues:
 //   logits^T[V,n] = Wt[V,H] * hidden[n,H]^T      (online-softmax statistics epilogue)
@@ -29,27 +32,21 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 #define MJ_DEV __device__ __forceinline__
 
 constexpr int kThreads = 256;
-constexpr int kBK = 32;              // K elements per LDS stage
-constexpr int kRowBytes = kBK * 2;   // 64 bytes per tile row in LDS
+constexpr int kBK = 64;              // K elements per LDS stage
+constexpr int kRowBytes = kBK * 2;   // 128 bytes per tile row in LDS
+constexpr int kSteps = kBK / 16;     // MFMA k-steps per stage
 constexpr uint32_t kOob = 0x7ffffff0u;   // byte offset that every descriptor below rejects
-
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 MJ_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
   // raw buffer (stride 0), 32-bit data format word for gfx9-class descriptors
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
 }
 
-// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding: vmcnt = [15:14|3:0]).
-template <int N>
-MJ_DEV void wait_vmcnt() {
-  static_assert(N >= 0 && N < 64, "vmcnt is 6 bits");
-  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
-}
+// s_waitcnt with only the LDS/scalar counter constrained (gfx9 encoding).
 MJ_DEV void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc07f); }
 
-// Position of 16-byte chunk c of tile row r inside the row's 64 bytes.
-MJ_DEV int swz(int r) { return ((r >> 1) & 3) ^ ((r >> 3) & 1); }
+// Chunk c of tile row r lives at 16-byte slot c ^ swz(r) of the row's 128 bytes.
+MJ_DEV int swz(int r) { return (r ^ (r >> 3)) & 7; }
 
 // Maps a linear workgroup id to a tile so that (a) the 32 workgroups that land on one
 // XCD at a time (ids congruent mod 8 go to the same XCD) form a GM x GN block of tiles
@@ -73,17 +70,16 @@ struct TileMap {
   }
 };
 
-template <int BM, int BN, int STAGES = 4>
+template <int BM, int BN>
 struct GemmTN {
-  static_assert(BM % 64 == 0 && BN % 64 == 0, "tile sides are multiples of 64");
+  static_assert(BM % 32 == 0 && BN % 32 == 0, "tile sides are multiples of 32");
   static constexpr int WM = BM / 2, WN = BN / 2;     // wavefront tile
   static constexpr int MI = WM / 32, NI = WN / 32;   // 32x32 blocks per wavefront
-  static constexpr int A_LD = BM / 64, B_LD = BN / 64;   // 16-byte loads per thread per stage
+  static constexpr int A_LD = BM / 32, B_LD = BN / 32;   // 16-byte loads per thread per stage
   static constexpr int LPS = A_LD + B_LD;
   static constexpr int kStageBytes = (BM + BN) * kRowBytes;
-  static constexpr int kLdsBytes = STAGES * kStageBytes;
+  static constexpr int kLdsBytes = 2 * kStageBytes;
   static_assert(kLdsBytes <= 160 * 1024, "LDS is 160 KB per CU");
-  static_assert((STAGES - 1) * LPS < 64, "outstanding loads must fit the vmcnt counter");
 
   // acc[mi][ni][r]: row = mi*32 + (r/4)*8 + (lane/32)*4 + r%4, col = ni*32 + lane%32
   // within the wavefront tile whose origin is (wm*WM, wn*WN).
@@ -102,65 +98,71 @@ struct GemmTN {
     const __amdgpu_buffer_rsrc_t ra = make_rsrc(A, bytes_a);
     const __amdgpu_buffer_rsrc_t rb = make_rsrc(B, bytes_b);
 
-    // Direct-to-LDS copy: one instruction of one wavefront fills 1024 contiguous LDS bytes
-    // (16 tile rows), lane -> (row = lane/4, slot = lane%4); the lane fetches global chunk
-    // slot ^ swz(row) so the LDS image is the swizzled one.
-    const int ld_row = wave * 16 + (lane >> 2);              // + 64*i
-    const int ld_chunk = (lane & 3) ^ swz(lane >> 2);        // row base is a multiple of 16
+    // Global -> register staging: thread t fetches chunk t%8 of tile rows t/8 + 32*i.
+    const int ld_row = t >> 3, ld_chunk = t & 7;
     uint32_t goff_a[A_LD], goff_b[B_LD];
 #pragma unroll
-    for (int i = 0; i < A_LD; ++i) goff_a[i] = (uint32_t)((ld_row + 64 * i) * lda * 2 + ld_chunk * 16);
+    for (int i = 0; i < A_LD; ++i) goff_a[i] = (uint32_t)((ld_row + 32 * i) * lda * 2 + ld_chunk * 16);
 #pragma unroll
-    for (int i = 0; i < B_LD; ++i) goff_b[i] = (uint32_t)((ld_row + 64 * i) * ldb * 2 + ld_chunk * 16);
+    for (int i = 0; i < B_LD; ++i) goff_b[i] = (uint32_t)((ld_row + 32 * i) * ldb * 2 + ld_chunk * 16);
     const int klimit = K - ld_chunk * 8;   // chunk is inside the row iff k0 < klimit
+    // swz(row + 32*i) == swz(row): one LDS write offset serves every i
+    const int st_off = ld_row * kRowBytes + ((ld_chunk ^ swz(ld_row)) << 4);
 
-    auto issue = [&](int slice) {
+    u32x4 stage[LPS];
+    // Load j (of the LPS this thread issues per slice).  Branch-free: a chunk at or beyond K
+    // (K tail, or a whole slice past the end) is redirected to an offset the descriptor rejects.
+    auto load_one = [&](int slice, int j) {
       const int k0 = slice * kBK;
-      char* base = smem + (slice % STAGES) * kStageBytes + wave * 1024;
-      if (k0 + kBK <= K) {
-#pragma unroll
-        for (int i = 0; i < A_LD; ++i)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * 4096), 16, goff_a[i], k0 * 2, 0, 0);
-#pragma unroll
-        for (int i = 0; i < B_LD; ++i)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(base + BM * kRowBytes + i * 4096), 16,
-                                                   goff_b[i], k0 * 2, 0, 0);
-      } else {   // K tail (or past the end): chunks at or beyond K read as zero
-        const bool in = k0 < klimit;
-#pragma unroll
-        for (int i = 0; i < A_LD; ++i)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * 4096), 16,
-                                                   in ? goff_a[i] + k0 * 2 : kOob, 0, 0, 0);
-#pragma unroll
-        for (int i = 0; i < B_LD; ++i)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(base + BM * kRowBytes + i * 4096), 16,
-                                                   in ? goff_b[i] + k0 * 2 : kOob, 0, 0, 0);
-      }
+      const bool in = k0 < klimit;
+      if (j < A_LD)
+        stage[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, in ? goff_a[j] : kOob, k0 * 2, 0);
+      else
+        stage[j] = __builtin_amdgcn_raw_buffer_load_b128(rb, in ? goff_b[j - A_LD] : kOob, k0 * 2, 0);
+    };
+    auto store_one = [&](int slice, int j) {
+      char* base = smem + (slice & 1) * kStageBytes + st_off;
+      if (j < A_LD)
+        *(u32x4*)(base + j * 32 * kRowBytes) = stage[j];
+      else
+        *(u32x4*)(base + BM * kRowBytes + (j - A_LD) * 32 * kRowBytes) = stage[j];
     };
 
     // LDS read positions: row within a 32-row block = lane % 32, k-chunk = 2*ks + lane/32
-    int rd_off[2];
+    int rd_off[kSteps];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) rd_off[ks] = l31 * kRowBytes + (((2 * ks + lhi) ^ swz(l31)) << 4);
+    for (int ks = 0; ks < kSteps; ++ks) rd_off[ks] = l31 * kRowBytes + (((2 * ks + lhi) ^ swz(l31)) << 4);
     const int a_base = wm * WM * kRowBytes;
     const int b_base = BM * kRowBytes + wn * WN * kRowBytes;
 
     bf16x8 fa[2][MI], fb[2][NI];
-    auto read_frags = [&](int slice, int ks, int buf) {
-      const char* sbase = smem + (slice % STAGES) * kStageBytes;
-#pragma unroll
-      for (int mi = 0; mi < MI; ++mi)
-        fa[buf][mi] = *(const bf16x8*)(sbase + a_base + mi * 32 * kRowBytes + rd_off[ks]);
-#pragma unroll
-      for (int ni = 0; ni < NI; ++ni)
-        fb[buf][ni] = *(const bf16x8*)(sbase + b_base + ni * 32 * kRowBytes + rd_off[ks]);
+    auto read_one = [&](int slice, int ks, int buf, int g) {   // fragment g of the MI + NI
+      const char* sbase = smem + (slice & 1) * kStageBytes;
+      if (g < MI)
+        fa[buf][g] = *(const bf16x8*)(sbase + a_base + g * 32 * kRowBytes + rd_off[ks]);
+      else
+        fb[buf][g - MI] = *(const bf16x8*)(sbase + b_base + (g - MI) * 32 * kRowBytes + rd_off[ks]);
     };
-    auto mma = [&](int buf) {
+    // One k-step, hand-scheduled: MI+NI groups, each = [LDS write of one staged chunk of the next
+    // slice, then the global load that refills that staging register with the slice after it]
+    // + one LDS read of the next k-step's fragments + this k-step's share of MFMAs.  The fences
+    // keep the groups in this order, so the MFMA pipe always has work queued behind every memory
+    // instruction.  `first` is the index of this k-step's first staged chunk (>= LPS: none left).
+    constexpr int G = MI + NI, T = MI * NI;
+    auto kstep = [&](int buf, int next_slice, int next_ks, int kt, int first) {
 #pragma unroll
-      for (int mi = 0; mi < MI; ++mi)
+      for (int g = 0; g < G; ++g) {
+        if (first + g < LPS) {
+          store_one(kt + 1, first + g);
+          load_one(kt + 2, first + g);
+        }
+        read_one(next_slice, next_ks, buf ^ 1, g);
 #pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][mi], fb[buf][ni], acc[mi][ni], 0, 0, 0);
+        for (int p = g * T / G; p < (g + 1) * T / G; ++p)
+          acc[p / NI][p % NI] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][p / NI], fb[buf][p % NI],
+                                                                        acc[p / NI][p % NI], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     };
 
 #pragma unroll
@@ -170,23 +172,29 @@ struct GemmTN {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
 
+    static_assert(LPS <= 3 * G, "the staged chunks of a slice must fit the first three k-steps");
     const int KT = (K + kBK - 1) / kBK;
 #pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) issue(s);
-    wait_vmcnt<(STAGES - 2) * LPS>();   // slice 0 has landed (this wavefront's part)
-    __builtin_amdgcn_s_barrier();       // ... and everyone else's
-    read_frags(0, 0, 0);
-    for (int kt = 0; kt < KT; ++kt) {
-      issue(kt + STAGES - 1);           // into the stage that slice kt-1 occupied
-      read_frags(kt, 1, 1);
-      mma(0);
-      wait_lgkmcnt0();                  // this wavefront is done reading slice kt
-      wait_vmcnt<(STAGES - 2) * LPS>(); // slice kt+1 has landed
-      __builtin_amdgcn_s_barrier();
-      read_frags(kt + 1, 0, 0);
-      mma(1);
+    for (int j = 0; j < LPS; ++j) load_one(0, j);
+#pragma unroll
+    for (int j = 0; j < LPS; ++j) {
+      store_one(0, j);
+      load_one(1, j);
     }
-    wait_vmcnt<0>();                    // drain the (empty) prefetches before LDS is reused
+    wait_lgkmcnt0();
+    __builtin_amdgcn_s_barrier();       // slice 0 is in LDS, slice 1 is on its way to the registers
+#pragma unroll
+    for (int g = 0; g < G; ++g) read_one(0, 0, 0, g);
+    for (int kt = 0; kt < KT; ++kt) {
+      // slice kt+1 moves registers -> the stage slice kt-1 occupied; slice kt+2 starts loading
+      kstep(0, kt, 1, kt, 0);
+      kstep(1, kt, 2, kt, G);
+      kstep(0, kt, 3, kt, 2 * G);
+      wait_lgkmcnt0();                  // own reads of slice kt and writes of slice kt+1 are done
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      kstep(1, kt + 1, 0, kt, LPS);
+    }
   }
 };
 
