@@ -19,7 +19,7 @@
  * old_logp[N] f32 or NULL (NULL = on-policy, ratio == 1, train_modules/__init__.py:161-165),
  * advantages[N] f32 (the reference's [B] broadcast per token, :173), mask[N] f32 in {0,1}.
  * Requirements: H % 8 == 0, V % 8 == 0, ld_hidden % 8 == 0, ld_w % 8 == 0,
- * bf16 pointers 16-byte aligned, temperature == 1.
+ * bf16 pointers, d_lm_head and the workspace 16-byte aligned, temperature == 1.
  */
 #ifndef MJ_GRPO_H
 #define MJ_GRPO_H
@@ -113,15 +113,14 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
  * per kernel id, the summed duration in milliseconds and the number of launches.  Process-wide
  * and not thread-safe: use from one thread. */
 enum {
-  MJ_GRPO_K_TRANSPOSE = 0,
-  MJ_GRPO_K_TARGET_LOGIT = 1,
-  MJ_GRPO_K_LOGITS_STATS = 2,
-  MJ_GRPO_K_FINALIZE = 3,
-  MJ_GRPO_K_DZ = 4,
-  MJ_GRPO_K_DHIDDEN = 5,
-  MJ_GRPO_K_DW = 6,
-  MJ_GRPO_K_REDUCE_LOSS = 7,
-  MJ_GRPO_K_COUNT = 8
+  MJ_GRPO_K_LOGITS_STATS = 0,
+  MJ_GRPO_K_FINALIZE = 1,
+  MJ_GRPO_K_DZ = 2,
+  MJ_GRPO_K_DHIDDEN = 3,
+  MJ_GRPO_K_DHIDDEN_REDUCE = 4,
+  MJ_GRPO_K_DW = 5,
+  MJ_GRPO_K_REDUCE_LOSS = 6,
+  MJ_GRPO_K_COUNT = 7
 };
 int mj_grpo_profile_begin(int max_launches);
 int mj_grpo_profile_end(double* total_ms /* [MJ_GRPO_K_COUNT] */, int* launches /* [MJ_GRPO_K_COUNT] */);

@@ -17,8 +17,8 @@ FLAG_SFT = 1 << 1
 EXPORTS = ("mj_grpo_version", "mj_grpo_last_error", "mj_grpo_workspace_bytes", "mj_grpo_forward",
            "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_profile_begin", "mj_grpo_profile_end")
 
-KERNEL_NAMES = ("k_transpose_bf16", "k_target_logit", "k_logits_stats", "k_finalize", "k_dz", "k_dhidden",
-                "k_dw", "k_reduce_loss")
+KERNEL_NAMES = ("k_logits_stats", "k_finalize", "k_dz", "k_dhidden", "k_dhidden_reduce", "k_dw",
+                "k_reduce_loss")
 
 
 class MjGrpoDesc(C.Structure):

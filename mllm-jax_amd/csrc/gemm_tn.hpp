@@ -1,24 +1,27 @@
 // gemm_tn.hpp -- bf16 MFMA tile engine for gfx950 (CDNA4), wave64.
 //
-// C[M,N] (fp32 accumulators) = A[M,K] * B[N,K]^T, both operands K-contiguous ("TN").
-// One workgroup of 256 threads (4 wavefronts, 2x2) owns a BM x BN tile; each wavefront owns
-// (BM/2) x (BN/2) as a grid of 32x32 MFMA blocks (v_mfma_f32_32x32x16_bf16).
+// C[M,N] (fp32 accumulators) = sum_k A(m,k) * B(n,k).  One workgroup of 256 threads
+// (4 wavefronts, 2x2) owns a BM x BN tile; each wavefront owns (BM/2) x (BN/2) as a grid of
+// 32x32 MFMA blocks (v_mfma_f32_32x32x16_bf16).
+//
+// Each operand may live in memory in either of two layouts, so no operand ever needs a
+// transposed copy:
+//   kRowK : X[row][k], k contiguous  -- LDS image 128 bytes per tile row, MFMA fragments come
+//           out with one ds_read_b128 per lane;
+//   kKRow : X[k][row], rows contiguous -- LDS image 64 k-rows of 2*ROWS bytes, MFMA fragments
+//           come out of two ds_read_b64_tr_b16 (the LDS transposing read of gfx950).
+// Both give lane l of a fragment the same k order (8*(l/32) + 0..7), so they mix freely.
 //
 // K is walked in slices of 64 through two LDS stages.  A slice travels global memory ->
-// registers (16-byte buffer loads, every 8 lanes cover one full 128-byte line of a tile row) ->
-// LDS (ds_write_b128) -> MFMA operands (ds_read_b128).  The loads of slice k+2 and the LDS writes
-// of slice k+1 are issued one at a time between the MFMAs of slice k, so the texture-address unit
-// sees an even trickle instead of a burst and every load has a whole slice of math to land.  Rows
-// past the operand's end read as zero through the buffer descriptor's range check; K tails are
-// masked per 16-byte chunk.  The LDS image of a slice is 128 bytes per row; 16-byte chunk c of
-// row r sits at slot c ^ swz(r), which keeps both the writes and the ds_read_b128 of consecutive
-// rows bank-conflict free whether the LDS serves 8 or 16 lanes per clock.  MFMA operands are
-// double-buffered in registers: the LDS reads of k-step s+1 sit between the MFMAs of k-step s.
-//
-// The three contractions of the loss path are instances of this engine with different epilogues:
-//   logits^T[V,n] = Wt[V,H] * hidden[n,H]^T      (online-softmax statistics epilogue)
-//   dHidden[n,H]  = dZ[n,V] * W[H,V]^T
-//   dW[H,V]       = hiddenT[H,n] * dZt[V,n]^T
+// registers (16-byte buffer loads that cover whole 128-byte lines) -> LDS (ds_write_b128) ->
+// MFMA operands.  The loads of slice k+2 and the LDS writes of slice k+1 are issued one at a
+// time between the MFMAs of slice k, so the texture-address unit and the LDS see an even
+// trickle instead of bursts and every load has a whole slice of math to land.  Rows / k-rows
+// past the operand's end read as zero through the buffer descriptor's range check; tails in
+// the contiguous direction are masked per 16-byte chunk.  16-byte chunks are XOR-permuted
+// inside their LDS row so that the writes and both kinds of fragment read are bank-conflict
+// free.  MFMA operands are double-buffered in registers: the LDS reads of k-step s+1 sit
+// between the MFMAs of k-step s.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -27,26 +30,28 @@ namespace mj {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
 
 #define MJ_DEV __device__ __forceinline__
 
 constexpr int kThreads = 256;
 constexpr int kBK = 64;              // K elements per LDS stage
-constexpr int kRowBytes = kBK * 2;   // 128 bytes per tile row in LDS
 constexpr int kSteps = kBK / 16;     // MFMA k-steps per stage
 constexpr uint32_t kOob = 0x7ffffff0u;   // byte offset that every descriptor below rejects
 
-MJ_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+enum Layout { kRowK = 0, kKRow = 1 };
+
+MJ_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
   // raw buffer (stride 0), 32-bit data format word for gfx9-class descriptors
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+  const int64_t capped = bytes < 0 ? 0 : (bytes > 0x7fffff00 ? 0x7fffff00 : bytes);
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)capped, 0x00020000);
 }
 
 // s_waitcnt with only the LDS/scalar counter constrained (gfx9 encoding).
 MJ_DEV void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc07f); }
-
-// Chunk c of tile row r lives at 16-byte slot c ^ swz(r) of the row's 128 bytes.
-MJ_DEV int swz(int r) { return (r ^ (r >> 3)) & 7; }
 
 // Maps a linear workgroup id to a tile so that (a) the 32 workgroups that land on one
 // XCD at a time (ids congruent mod 8 go to the same XCD) form a GM x GN block of tiles
@@ -56,10 +61,8 @@ struct TileMap {
   int tiles_m, tiles_n, sb_m, sb_n;
   __host__ __device__ TileMap(int tm, int tn)
       : tiles_m(tm), tiles_n(tn), sb_m((tm + GM - 1) / GM), sb_n((tn + GN - 1) / GN) {}
-  __host__ int grid() const {
-    int sb = sb_m * sb_n;
-    return ((sb + 7) / 8) * 8 * (GM * GN);
-  }
+  __host__ __device__ int items() const { return ((sb_m * sb_n + 7) / 8) * 8 * (GM * GN); }
+  __host__ int grid() const { return items(); }
   MJ_DEV bool tile(int pid, int& tm, int& tn) const {
     const int xcd = pid & 7, q = pid >> 3;
     const int sb = (q / (GM * GN)) * 8 + xcd, within = q % (GM * GN);
@@ -70,14 +73,115 @@ struct TileMap {
   }
 };
 
-template <int BM, int BN>
+// One operand of the tile: ROWS tile rows (M or N direction) by 64 k per slice, 128*ROWS bytes of
+// LDS per stage, ROWS/32 16-byte chunks per thread per slice.
+template <int ROWS, int LAYOUT>
+struct Operand {
+  static constexpr int LD = ROWS / 32;
+  static constexpr int kBytes = ROWS * 128;
+
+  const char* base;      // tile origin: (row 0, k 0)
+  int64_t ld2;           // bytes between consecutive rows (kRowK) / k-rows (kKRow)
+  int rows, K;           // valid rows of this tile, K extent
+  __amdgpu_buffer_rsrc_t rsrc;   // kRowK: whole tile; kKRow: current slice (see slice_begin)
+  uint32_t goff[LD];     // byte offset of this thread's chunk i inside the tile / slice
+  int st_off;            // LDS byte offset of chunk 0 (kRowK) ...
+  int st_off1;           // ... and of odd i for kKRow (bit 3 of the k-row enters the permutation)
+  int klimit;            // kRowK: chunk is inside the row iff k0 < klimit
+  bool col_ok;           // kKRow: this thread's chunk lies inside the valid rows
+  int rd[4];             // LDS read offsets: kRowK per k-step, kKRow per fragment
+
+  // 64-byte segment permutation of the kKRow image: 8 k-rows read by one transposing read
+  // ({r..r+3} and {r+8..r+11}) must land in 8 different segments of the 512-byte row.
+  static MJ_DEV int sigma(int krow) { return (krow & 3) | ((krow >> 1) & 4); }
+  // 16-byte chunk permutation of the kRowK image (see the file header).
+  static MJ_DEV int swz(int r) { return (r ^ (r >> 3)) & 7; }
+
+  MJ_DEV void init(const __bf16* p, int rows_valid, int64_t ld, int K_, int wave_row0) {
+    static_assert(LAYOUT == kRowK || ROWS == 256, "the k-major image is laid out for 256-row tiles");
+    const int t = threadIdx.x, lane = t & 63;
+    base = (const char*)p;
+    ld2 = ld * 2;
+    rows = rows_valid < ROWS ? rows_valid : ROWS;
+    K = K_;
+    if (LAYOUT == kRowK) {
+      const int row = t >> 3, chunk = t & 7;     // chunk t%8 of tile rows t/8 + 32*i
+      rsrc = make_rsrc(base, (int64_t)rows * ld2);
+#pragma unroll
+      for (int i = 0; i < LD; ++i) goff[i] = (uint32_t)((row + 32 * i) * ld2 + chunk * 16);
+      klimit = K - chunk * 8;
+      st_off = row * 128 + ((chunk ^ swz(row)) << 4);   // swz(row + 32*i) == swz(row)
+      st_off1 = st_off;
+      col_ok = true;
+      const int l31 = lane & 31, lhi = lane >> 5;       // fragment row, k-chunk 2*ks + lane/32
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+        rd[ks] = (wave_row0 + l31) * 128 + (((2 * ks + lhi) ^ swz(l31)) << 4);
+    } else {
+      constexpr int CPR = ROWS / 8;              // 16-byte chunks per k-row
+      const int krow = t / CPR, chunk = t % CPR; // chunk of k-rows krow + 8*i
+#pragma unroll
+      for (int i = 0; i < LD; ++i) goff[i] = (uint32_t)((krow + (256 / CPR) * i) * ld2 + chunk * 16);
+      col_ok = chunk * 8 < rows;
+      klimit = 0;
+      st_off = krow * (ROWS * 2) + ((chunk ^ (sigma(krow) << 2)) << 4);
+      st_off1 = krow * (ROWS * 2) + ((chunk ^ (sigma(krow + 8) << 2)) << 4);
+      // Transposing read: the 16 lanes of a group fetch 4 k-rows x 4 row-quads (8 bytes each) and
+      // get back, lane i, the 4 k of row i.  Lane l: group g = l/16, s = l%16 reads k-row
+      // (g/2)*8 + s/4 (+4 for the second read, +16*ks), quad (g%2)*4 + s%4 of the 32-row fragment.
+      const int g = lane >> 4, s = lane & 15;
+      const int kr = (g >> 1) * 8 + (s >> 2);
+#pragma unroll
+      for (int f = 0; f < 4; ++f) {
+        const int quad = (wave_row0 + f * 32) / 4 + (g & 1) * 4 + (s & 3);
+        rd[f] = kr * (ROWS * 2) + ((((quad >> 1) ^ (sigma(kr) << 2))) << 4) + (quad & 1) * 8;
+      }
+    }
+  }
+
+  // kKRow: point the descriptor at slice `slice` (its k-rows past K fall outside and read zero).
+  MJ_DEV void slice_begin(int slice) {
+    if (LAYOUT == kKRow) {
+      const int k0 = slice * kBK;
+      const int left = K - k0;
+      rsrc = make_rsrc(base + (int64_t)k0 * ld2, (int64_t)(left < kBK ? left : kBK) * ld2);
+    }
+  }
+  MJ_DEV u32x4 load(int slice, int i) const {
+    if (LAYOUT == kRowK) {
+      const int k0 = slice * kBK;
+      return __builtin_amdgcn_raw_buffer_load_b128(rsrc, k0 < klimit ? goff[i] : kOob, k0 * 2, 0);
+    }
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, col_ok ? goff[i] : kOob, 0, 0);
+  }
+  MJ_DEV void store(char* stage, int i, u32x4 v) const {
+    if (LAYOUT == kRowK)
+      *(u32x4*)(stage + st_off + i * 32 * 128) = v;
+    else
+      *(u32x4*)(stage + ((i & 1) ? st_off1 : st_off) + i * 8 * (ROWS * 2)) = v;
+  }
+  // MFMA fragment f (32 rows) of k-step ks.
+  MJ_DEV bf16x8 frag(const char* stage, int f, int ks) const {
+    if (LAYOUT == kRowK) return *(const bf16x8*)(stage + rd[ks] + f * 32 * 128);
+    typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+    const char* p = stage + rd[f] + ks * 16 * (ROWS * 2);
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * (ROWS * 2)));
+    const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, v);
+  }
+};
+
+template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK>
 struct GemmTN {
   static_assert(BM % 32 == 0 && BN % 32 == 0, "tile sides are multiples of 32");
   static constexpr int WM = BM / 2, WN = BN / 2;     // wavefront tile
   static constexpr int MI = WM / 32, NI = WN / 32;   // 32x32 blocks per wavefront
-  static constexpr int A_LD = BM / 32, B_LD = BN / 32;   // 16-byte loads per thread per stage
-  static constexpr int LPS = A_LD + B_LD;
-  static constexpr int kStageBytes = (BM + BN) * kRowBytes;
+  using OpA = Operand<BM, LAY_A>;
+  using OpB = Operand<BN, LAY_B>;
+  static constexpr int A_LD = OpA::LD, B_LD = OpB::LD;
+  static constexpr int LPS = A_LD + B_LD;            // 16-byte chunks per thread per slice
+  static constexpr int kStageBytes = OpA::kBytes + OpB::kBytes;
   static constexpr int kLdsBytes = 2 * kStageBytes;
   static_assert(kLdsBytes <= 160 * 1024, "LDS is 160 KB per CU");
 
@@ -85,69 +189,38 @@ struct GemmTN {
   // within the wavefront tile whose origin is (wm*WM, wn*WN).
   f32x16 acc[MI][NI];
 
-  // A: tile origin pointer (row m0, k 0), rows_a valid rows, lda elements; same for B.
+  // A, B: tile origin pointers (row 0 of the tile, k = k_begin); rows_*: valid rows of the tile;
+  // ld*: elements between rows (kRowK) or between k-rows (kKRow); K: k extent from the origin.
   MJ_DEV void run(const __bf16* A, int rows_a, int64_t lda, const __bf16* B, int rows_b,
                   int64_t ldb, int K, char* smem) {
-    const int t = threadIdx.x;
-    const int lane = t & 63, wave = t >> 6;
+    const int wave = threadIdx.x >> 6;
     const int wm = wave & 1, wn = wave >> 1;
-    const int l31 = lane & 31, lhi = lane >> 5;
+    OpA a;
+    OpB b;
+    a.init(A, rows_a, lda, K, wm * WM);
+    b.init(B, rows_b, ldb, K, wn * WN);
 
-    const uint32_t bytes_a = (uint32_t)min((int64_t)min(rows_a, BM) * lda * 2, (int64_t)0x7fffff00);
-    const uint32_t bytes_b = (uint32_t)min((int64_t)min(rows_b, BN) * ldb * 2, (int64_t)0x7fffff00);
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc(A, bytes_a);
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(B, bytes_b);
-
-    // Global -> register staging: thread t fetches chunk t%8 of tile rows t/8 + 32*i.
-    const int ld_row = t >> 3, ld_chunk = t & 7;
-    uint32_t goff_a[A_LD], goff_b[B_LD];
-#pragma unroll
-    for (int i = 0; i < A_LD; ++i) goff_a[i] = (uint32_t)((ld_row + 32 * i) * lda * 2 + ld_chunk * 16);
-#pragma unroll
-    for (int i = 0; i < B_LD; ++i) goff_b[i] = (uint32_t)((ld_row + 32 * i) * ldb * 2 + ld_chunk * 16);
-    const int klimit = K - ld_chunk * 8;   // chunk is inside the row iff k0 < klimit
-    // swz(row + 32*i) == swz(row): one LDS write offset serves every i
-    const int st_off = ld_row * kRowBytes + ((ld_chunk ^ swz(ld_row)) << 4);
-
-    u32x4 stage[LPS];
-    // Load j (of the LPS this thread issues per slice).  Branch-free: a chunk at or beyond K
-    // (K tail, or a whole slice past the end) is redirected to an offset the descriptor rejects.
+    u32x4 staged[LPS];
     auto load_one = [&](int slice, int j) {
-      const int k0 = slice * kBK;
-      const bool in = k0 < klimit;
-      if (j < A_LD)
-        stage[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, in ? goff_a[j] : kOob, k0 * 2, 0);
-      else
-        stage[j] = __builtin_amdgcn_raw_buffer_load_b128(rb, in ? goff_b[j - A_LD] : kOob, k0 * 2, 0);
+      if (j < A_LD) staged[j] = a.load(slice, j);
+      else staged[j] = b.load(slice, j - A_LD);
     };
     auto store_one = [&](int slice, int j) {
-      char* base = smem + (slice & 1) * kStageBytes + st_off;
-      if (j < A_LD)
-        *(u32x4*)(base + j * 32 * kRowBytes) = stage[j];
-      else
-        *(u32x4*)(base + BM * kRowBytes + (j - A_LD) * 32 * kRowBytes) = stage[j];
+      char* stage = smem + (slice & 1) * kStageBytes;
+      if (j < A_LD) a.store(stage, j, staged[j]);
+      else b.store(stage + OpA::kBytes, j - A_LD, staged[j]);
     };
-
-    // LDS read positions: row within a 32-row block = lane % 32, k-chunk = 2*ks + lane/32
-    int rd_off[kSteps];
-#pragma unroll
-    for (int ks = 0; ks < kSteps; ++ks) rd_off[ks] = l31 * kRowBytes + (((2 * ks + lhi) ^ swz(l31)) << 4);
-    const int a_base = wm * WM * kRowBytes;
-    const int b_base = BM * kRowBytes + wn * WN * kRowBytes;
-
     bf16x8 fa[2][MI], fb[2][NI];
     auto read_one = [&](int slice, int ks, int buf, int g) {   // fragment g of the MI + NI
-      const char* sbase = smem + (slice & 1) * kStageBytes;
-      if (g < MI)
-        fa[buf][g] = *(const bf16x8*)(sbase + a_base + g * 32 * kRowBytes + rd_off[ks]);
-      else
-        fb[buf][g - MI] = *(const bf16x8*)(sbase + b_base + (g - MI) * 32 * kRowBytes + rd_off[ks]);
+      const char* stage = smem + (slice & 1) * kStageBytes;
+      if (g < MI) fa[buf][g] = a.frag(stage, g, ks);
+      else fb[buf][g - MI] = b.frag(stage + OpA::kBytes, g - MI, ks);
     };
     // One k-step, hand-scheduled: MI+NI groups, each = [LDS write of one staged chunk of the next
     // slice, then the global load that refills that staging register with the slice after it]
-    // + one LDS read of the next k-step's fragments + this k-step's share of MFMAs.  The fences
-    // keep the groups in this order, so the MFMA pipe always has work queued behind every memory
-    // instruction.  `first` is the index of this k-step's first staged chunk (>= LPS: none left).
+    // + the LDS read of one of the next k-step's fragments + this k-step's share of MFMAs.  The
+    // fences keep the groups in this order, so the MFMA pipe always has work queued behind every
+    // memory instruction.  `first` is the index of this k-step's first staged chunk (>= LPS: none).
     constexpr int G = MI + NI, T = MI * NI;
     auto kstep = [&](int buf, int next_slice, int next_ks, int kt, int first) {
 #pragma unroll
@@ -174,8 +247,12 @@ struct GemmTN {
 
     static_assert(LPS <= 3 * G, "the staged chunks of a slice must fit the first three k-steps");
     const int KT = (K + kBK - 1) / kBK;
+    a.slice_begin(0);
+    b.slice_begin(0);
 #pragma unroll
     for (int j = 0; j < LPS; ++j) load_one(0, j);
+    a.slice_begin(1);
+    b.slice_begin(1);
 #pragma unroll
     for (int j = 0; j < LPS; ++j) {
       store_one(0, j);
@@ -187,6 +264,8 @@ struct GemmTN {
     for (int g = 0; g < G; ++g) read_one(0, 0, 0, g);
     for (int kt = 0; kt < KT; ++kt) {
       // slice kt+1 moves registers -> the stage slice kt-1 occupied; slice kt+2 starts loading
+      a.slice_begin(kt + 2);
+      b.slice_begin(kt + 2);
       kstep(0, kt, 1, kt, 0);
       kstep(1, kt, 2, kt, G);
       kstep(0, kt, 3, kt, 2 * G);

@@ -51,10 +51,26 @@ constexpr int64_t kDefaultChunk = 8192;    // tokens whose logits live in the wo
 inline int64_t rup(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 
 struct Plan {
-  int64_t N, H, V, chunk, n_pad, parts, ld_ht;
+  int64_t N, H, V, chunk, n_pad, parts;
+  int dh_splits;          // vocab splits of the dHidden product (1 = none)
+  int64_t dh_k_per_split;
   // byte offsets into the workspace
-  size_t wt, zy, term, pm, pl, ps, g, ht, zt, dz, total_fwd, total_bwd;
+  size_t zy, term, pm, pl, ps, g, zt, part, total_fwd, total_bwd;
 };
+
+// Splits of the dHidden product over the vocab: its (n/256) x (H/256) tiles rarely fill the 256
+// CUs in whole rounds, so K = V is cut into the fewest pieces (<= 8) that waste < 4% of a round.
+int pick_splits(int64_t tiles) {
+  int best = 1;
+  double best_eff = 0.0;
+  for (int s = 1; s <= 8; ++s) {
+    const int64_t items = tiles * s, rounds = (items + 255) / 256;
+    const double eff = (double)items / (double)(rounds * 256);
+    if (eff > best_eff + 1e-9) { best_eff = eff; best = s; }
+    if (eff >= 0.96) return s;
+  }
+  return best;
+}
 
 int make_plan(const MjGrpoDesc* d, Plan* p) {
   if (d == nullptr) return fail(MJ_GRPO_ERR_NULL, "desc is NULL");
@@ -78,13 +94,11 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   if (chunk > p->N) chunk = p->N;
   p->chunk = chunk;
   p->n_pad = rup(chunk, 256);
-  if (p->n_pad * p->V * 2 > (int64_t)0xffffffff)
-    return fail(MJ_GRPO_ERR_SHAPE, "chunk_tokens * vocab too large for one chunk; lower chunk_tokens");
   p->parts = 2 * ((p->V + BM - 1) / BM);
-  p->ld_ht = rup(p->N, 64);
+  p->dh_splits = pick_splits((p->n_pad / BM) * ((p->H + BN - 1) / BN));
+  p->dh_k_per_split = rup((p->V + p->dh_splits - 1) / p->dh_splits, 64);
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t at = o; o = (size_t)rup((int64_t)(o + bytes), 256); return at; };
-  p->wt = take((size_t)p->V * p->H * 2);
   p->zy = take((size_t)p->N * 4);
   p->term = take((size_t)p->N * 4);
   p->pm = take((size_t)p->parts * p->n_pad * 4);
@@ -92,9 +106,8 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   p->ps = take((size_t)p->parts * p->n_pad * 4);
   p->g = take((size_t)p->n_pad * 4);
   p->total_fwd = o;
-  p->ht = take((size_t)p->H * p->ld_ht * 2);
   p->zt = take((size_t)p->V * p->n_pad * 2);
-  p->dz = take((size_t)p->n_pad * p->V * 2);
+  p->part = take(p->dh_splits > 1 ? (size_t)p->dh_splits * p->n_pad * p->H * 4 : 0);
   p->total_bwd = o;
   return MJ_GRPO_OK;
 }
@@ -137,22 +150,21 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
   if (!workspace) return fail(MJ_GRPO_ERR_WORKSPACE, "workspace is NULL");
   const size_t need = bwd ? p.total_bwd : p.total_fwd;
   if (ws_bytes < need) return fail(MJ_GRPO_ERR_WORKSPACE, "workspace too small: %zu < %zu bytes", ws_bytes, need);
-  if (misaligned(hidden) || misaligned(lm_head) || misaligned(workspace) || (bwd && misaligned(d_hidden)))
-    return fail(MJ_GRPO_ERR_ALIGN, "hidden, lm_head, d_hidden and workspace must be 16-byte aligned");
+  if (misaligned(hidden) || misaligned(lm_head) || misaligned(workspace) ||
+      (bwd && (misaligned(d_hidden) || misaligned(d_w))))
+    return fail(MJ_GRPO_ERR_ALIGN, "hidden, lm_head, d_hidden, d_lm_head and workspace must be 16-byte aligned");
 
   hipStream_t st = (hipStream_t)stream_v;
   char* ws = (char*)workspace;
   const int N = (int)p.N, H = (int)p.H, V = (int)p.V;
-  __bf16* wt = (__bf16*)(ws + p.wt);
   float* zy = (float*)(ws + p.zy);
   float* term = (float*)(ws + p.term);
   float* pm = (float*)(ws + p.pm);
   float* pl = (float*)(ws + p.pl);
   float* ps = (float*)(ws + p.ps);
   float* g = (float*)(ws + p.g);
-  __bf16* ht = (__bf16*)(ws + p.ht);
   uint16_t* zt = (uint16_t*)(ws + p.zt);
-  uint16_t* dz = (uint16_t*)(ws + p.dz);
+  float* part = (float*)(ws + p.part);
   const float gscale = d->grad_loss_scale;
   const size_t lds = mj::GemmTN<BM, BN>::kLdsBytes;
 
@@ -162,34 +174,17 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     if ((rc = enable_lds(mj::k_dw<BM, BN>))) return rc;
   }
 
-  // lm_head[H,V] -> Wt[V,H]: K-contiguous operand of the logits product
-  {
-    Timed t(MJ_GRPO_K_TRANSPOSE, st);
-    mj::k_transpose_bf16<<<dim3((H + 63) / 64, (V + 63) / 64), 256, 0, st>>>(
-        (const uint16_t*)lm_head, d->ld_w, (uint16_t*)wt, H, H, V, H);
-  }
-  if (bwd) {   // hidden[N,H] -> hiddenT[H, ld_ht]: K-contiguous operand of the dW product
-    Timed t(MJ_GRPO_K_TRANSPOSE, st);
-    mj::k_transpose_bf16<<<dim3((unsigned)(p.ld_ht / 64), (H + 63) / 64), 256, 0, st>>>(
-        (const uint16_t*)hidden, d->ld_hidden, (uint16_t*)ht, p.ld_ht, N, H, (int)p.ld_ht);
-  }
-  if (mode != kBackwardOnly) {
-    Timed t(MJ_GRPO_K_TARGET_LOGIT, st);
-    mj::k_target_logit<<<(N + 3) / 4, 256, 0, st>>>((const __bf16*)hidden, d->ld_hidden, wt, H, targets, N,
-                                                    H, V, d->softcap, zy);
-  }
-  if ((rc = check_launch("prologue kernels"))) return rc;
-
   for (int64_t c0 = 0; c0 < p.N; c0 += p.chunk) {
     const int nc = (int)((p.N - c0 < p.chunk) ? p.N - c0 : p.chunk);
     const int n_pad = (int)rup(nc, 256);
     const __bf16* hid_c = (const __bf16*)hidden + c0 * d->ld_hidden;
     {
       mj::LogitsArgs a;
-      a.wt = wt; a.hid = hid_c; a.ld_wt = H; a.ld_hid = d->ld_hidden;
+      a.w = (const __bf16*)lm_head; a.hid = hid_c; a.ld_w = d->ld_w; a.ld_hid = d->ld_hidden;
       a.V = V; a.n = nc; a.H = H; a.cap = d->softcap;
       a.zt = bwd ? zt : nullptr; a.ld_z = p.n_pad;
       a.pm = pm; a.pl = pl; a.ps = ps; a.ld_p = p.n_pad;
+      a.targets = targets + c0; a.zy = zy + c0;
       mj::TileMap<4, 8> map((V + BM - 1) / BM, (nc + BN - 1) / BN);
       Timed t(MJ_GRPO_K_LOGITS_STATS, st);
       mj::k_logits_stats<BM, BN><<<map.grid(), mj::kThreads, lds, st>>>(a, map);
@@ -214,30 +209,40 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     }
     if (bwd) {
       mj::DzArgs z;
-      z.zt = zt; z.ld_z = p.n_pad; z.dz = dz; z.ld_dz = V;
+      z.zt = zt; z.ld_z = p.n_pad;
       z.lse = (mode == kBackwardOnly ? saved_lse : lse) + c0; z.g = g; z.targets = targets + c0;
       z.V = V; z.n = nc; z.n_pad = n_pad; z.cap = d->softcap;
       {
         Timed t(MJ_GRPO_K_DZ, st);
-        mj::k_dz<<<dim3((V + 63) / 64, n_pad / 64), 256, 0, st>>>(z);
+        mj::k_dz<<<dim3(n_pad / 256, (V + 63) / 64), 256, 0, st>>>(z);
       }
 
+      // the split count was planned for a full chunk; a shorter last chunk keeps it (the partial
+      // buffer is sized for it) unless it has a single split anyway
       mj::DhArgs h;
-      h.dz = (const __bf16*)dz; h.w = (const __bf16*)lm_head; h.ld_dz = V; h.ld_w = d->ld_w;
-      h.n = nc; h.H = H; h.V = V;
+      h.dzt = (const __bf16*)zt; h.w = (const __bf16*)lm_head; h.ld_z = p.n_pad; h.ld_w = d->ld_w;
+      h.n = nc; h.n_pad = n_pad; h.H = H; h.V = V;
+      h.splits = p.dh_splits; h.k_per_split = (int)p.dh_k_per_split;
       h.dh = (uint16_t*)d_hidden + c0 * d->ld_hidden; h.ld_dh = d->ld_hidden;
+      h.part = part;
       mj::TileMap<4, 8> mh((nc + BM - 1) / BM, (H + BN - 1) / BN);
       {
         Timed t(MJ_GRPO_K_DHIDDEN, st);
-        mj::k_dhidden<BM, BN><<<mh.grid(), mj::kThreads, lds, st>>>(h, mh);
+        mj::k_dhidden<BM, BN><<<mh.grid() * h.splits, mj::kThreads, lds, st>>>(h, mh);
+      }
+      if (h.splits > 1) {
+        const int64_t work = (int64_t)nc * (H / 4);
+        Timed t(MJ_GRPO_K_DHIDDEN_REDUCE, st);
+        mj::k_dhidden_reduce<<<(unsigned)((work + 255) / 256), 256, 0, st>>>(part, h.splits, nc, n_pad, H, h.dh,
+                                                                           h.ld_dh);
       }
 
       mj::DwArgs w;
-      w.ht = ht + c0; w.dzt = (const __bf16*)zt; w.ld_ht = p.ld_ht; w.ld_z = p.n_pad;
-      w.H = H; w.V = V; w.K = (int)rup(nc, 8);
+      w.dzt = (const __bf16*)zt; w.hid = hid_c; w.ld_z = p.n_pad; w.ld_hid = d->ld_hidden;
+      w.H = H; w.V = V; w.n = nc;
       w.dw = d_w; w.ld_dw = d->ld_w;
       w.accumulate = (c0 > 0 || (d->flags & MJ_GRPO_FLAG_DW_ACCUMULATE)) ? 1 : 0;
-      mj::TileMap<4, 8> mw((H + BM - 1) / BM, (V + BN - 1) / BN);
+      mj::TileMap<4, 8> mw((V + BM - 1) / BM, (H + BN - 1) / BN);
       {
         Timed t(MJ_GRPO_K_DW, st);
         mj::k_dw<BM, BN><<<mw.grid(), mj::kThreads, lds, st>>>(w, mw);

@@ -1,15 +1,17 @@
 // mj_grpo_kernels.hpp -- device kernels of the fused GRPO loss path (gfx950).
 //
 // Per token chunk of n rows (n <= chunk_tokens):
-//   k_logits_stats  : logits^T tile = Wt * hidden^T on MFMA; epilogue applies the softcap,
-//                     reduces (max, sum exp, sum exp*z) per token over the tile's vocab rows
+//   k_logits_stats  : logits^T tile [vocab x tokens] = W^T * hidden^T on MFMA, W and hidden read in
+//                     place; the epilogue applies the softcap, reduces (max, sum exp, sum exp*z)
+//                     per token over the tile's vocab rows, picks out the sampled token's logit
 //                     and (training) stores the capped logits as IEEE half, transposed [V, n].
-//   k_target_logit  : z[t, y_t] = <hidden[t,:], Wt[y_t,:]> in fp32 (one wavefront per token).
-//   k_finalize      : merges the per-tile statistics -> lse, logp, entropy, ratio / clip /
-//                     min surrogate, per-token loss term and dloss/dlogp.
-//   k_dz            : dZt = g * (onehot - exp(z - lse)) * softcap', in place, plus the
-//                     token-major copy dZ[n, V] for the dHidden product.
-//   k_dhidden, k_dw : the two backward contractions.
+//   k_finalize      : merges the per-tile statistics -> lse, logp, entropy, ratio / clip / min
+//                     surrogate, per-token loss term and dloss/dlogp.
+//   k_dz            : in place, logits^T -> dZ^T = g * (onehot - exp(z - lse)) * softcap' (bf16).
+//   k_dhidden       : dHidden[n,H] = dZ * W^T  (dZ read k-major from dZ^T), optionally split over
+//                     the vocab into fp32 partial sums that k_dhidden_reduce adds up.
+//   k_dw            : dW^T tile [vocab x hidden] = dZ^T * hidden, written / accumulated into
+//                     dW[H,V] with 16-byte accesses.
 // Nothing here allocates; all buffers come from the caller's workspace.
 #pragma once
 #include "gemm_tn.hpp"
@@ -21,7 +23,6 @@ constexpr float kLog2e = 1.4426950408889634f;
 // fma(z, kLog2e, -max * kLog2e) is exactly 0 when a whole half-tile holds only stand-ins.
 constexpr float kNegBig = -0x1p100f;
 
-MJ_DEV float bf16_to_f32(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
 MJ_DEV uint16_t f32_to_bf16(float f) {   // round to nearest even; inputs are finite
   uint32_t u = __float_as_uint(f);
   u += 0x7fffu + ((u >> 16) & 1u);
@@ -43,31 +44,33 @@ MJ_DEV float softcap_apply(float z, float cap, float inv_cap) {
 
 // ----------------------------------------------------------------------------- logits + stats
 struct LogitsArgs {
-  const __bf16* wt;      // [V, H] (ld = ld_wt)
+  const __bf16* w;       // lm_head [H, ld_w]
   const __bf16* hid;     // chunk origin, [n, ld_hid]
-  int64_t ld_wt, ld_hid;
+  int64_t ld_w, ld_hid;
   int V, n, H;
   float cap;             // 0 = off
   uint16_t* zt;          // [V, ld_z] half logits^T of the chunk, or nullptr (forward only)
   int64_t ld_z;
   float *pm, *pl, *ps;   // per (vocab half-tile, token) partial max / sum e / sum e*z, ld = ld_p
   int64_t ld_p;
+  const int32_t* targets;   // chunk origin
+  float* zy;                // chunk origin: capped logit of the sampled token
 };
 
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap<4, 8> map) {
-  using G = GemmTN<BM, BN>;
+  using G = GemmTN<BM, BN, kKRow, kRowK>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   int tm, tn;
   if (!map.tile(blockIdx.x, tm, tn)) return;
   const int m0 = tm * BM, n0 = tn * BN;
   G g;
-  g.run(p.wt + (int64_t)m0 * p.ld_wt, p.V - m0, p.ld_wt, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0,
-        p.ld_hid, p.H, smem);
+  g.run(p.w + m0, p.V - m0, p.ld_w, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0, p.ld_hid, p.H, smem);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
-  const int vbase = m0 + wm * G::WM + lhi * 4;   // + mi*32 + (r/4)*8 + r%4
+  const int vwave = m0 + wm * G::WM;             // first vocab row of this wavefront
+  const int vbase = vwave + lhi * 4;             // + mi*32 + (r/4)*8 + r%4
   const bool tail = (m0 + BM > p.V);
   const float inv_cap = p.cap > 0.f ? 1.f / p.cap : 0.f;
 #pragma unroll
@@ -104,6 +107,23 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
       p.pl[o] = l;
       p.ps[o] = s;
     }
+    // The sampled token's logit: exactly one lane of one tile holds it.  Few wavefronts have a
+    // hit at all (32 tokens x 128 rows out of V), so the register search sits behind a vote.
+    {
+      int y = col < p.n ? p.targets[col] : -1;
+      y = y >= p.V ? p.V - 1 : y;
+      const int d = y - vwave;                       // row inside the wavefront's 128
+      const bool hit = y >= 0 && d >= 0 && d < G::WM && ((d >> 2) & 1) == lhi;
+      if (__any(hit)) {
+        const int flat = (d >> 5) * 16 + ((d >> 3) & 3) * 4 + (d & 3);   // mi*16 + r
+        float zy = 0.f;
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) zy = (flat == mi * 16 + r) ? g.acc[mi][ni][r] : zy;
+        if (hit) p.zy[col] = zy;
+      }
+    }
     if (p.zt != nullptr) {
 #pragma unroll
       for (int mi = 0; mi < G::MI; ++mi)
@@ -114,32 +134,6 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
         }
     }
   }
-}
-
-// ----------------------------------------------------------------------------- target logit
-// One wavefront per token: zy[t] = softcap(<hid[t,:], wt[y_t,:]>).
-__global__ __launch_bounds__(256) void k_target_logit(const __bf16* hid, int64_t ld_hid,
-                                                      const __bf16* wt, int64_t ld_wt,
-                                                      const int32_t* targets, int n, int H, int V,
-                                                      float cap, float* zy) {
-  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (t >= n) return;
-  int y = targets[t];
-  y = y < 0 ? 0 : (y >= V ? V - 1 : y);
-  const uint16_t* a = (const uint16_t*)hid + (int64_t)t * ld_hid;
-  const uint16_t* b = (const uint16_t*)wt + (int64_t)y * ld_wt;
-  float acc = 0.f;
-  for (int k = lane * 8; k < H; k += 512) {
-    const u32x4 av = *(const u32x4*)(a + k), bv = *(const u32x4*)(b + k);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      acc = fmaf(__uint_as_float(av[i] << 16), __uint_as_float(bv[i] << 16), acc);
-      acc = fmaf(__uint_as_float(av[i] & 0xffff0000u), __uint_as_float(bv[i] & 0xffff0000u), acc);
-    }
-  }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
-  if (lane == 0) zy[t] = cap > 0.f ? softcap_apply(acc, cap, 1.f / cap) : acc;
 }
 
 // ----------------------------------------------------------------------------- finalize
@@ -252,89 +246,80 @@ __global__ __launch_bounds__(1024) void k_reduce_loss(const float* term, int n, 
 struct DzArgs {
   uint16_t* zt;        // [V, ld_z] in: capped logits^T (half); out: dZ^T (bf16)
   int64_t ld_z;
-  uint16_t* dz;        // [n_pad, ld_dz] out: dZ token-major
-  int64_t ld_dz;
-  const float *lse, *g;    // chunk-local [n_pad] (lse valid for t < n)
+  const float *lse, *g;    // chunk-local (lse valid for t < n, g for t < n_pad)
   const int32_t* targets;  // chunk origin
   int V, n, n_pad;
   float cap;
 };
 
-// block: 64 vocab rows x 64 tokens
+// Streaming, in place.  Block = 256 tokens (32 threads x 8) by 64 vocab rows (8 row-lanes x 8
+// steps): every wavefront instruction moves two full 512-byte row segments, and the per-token
+// constants are loaded once per thread.  Tokens at or beyond n (chunk padding) become exact zeros.
 __global__ __launch_bounds__(256) void k_dz(DzArgs p) {
-  __shared__ uint16_t tile[64][72];   // [v][token], padded
-  const int v0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
-  const int tx = threadIdx.x & 7, ty = threadIdx.x >> 3;   // 8 token-octets x 32 rows
+  const int cx = threadIdx.x & 31, ry = threadIdx.x >> 5;
+  const int t0 = blockIdx.x * 256 + cx * 8;
+  const int v0 = blockIdx.y * 64;
+  if (t0 >= p.n_pad) return;
   const float inv_cap2 = p.cap > 0.f ? 1.f / (p.cap * p.cap) : 0.f;
   float lse[8], g[8];
   int y[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int t = t0 + tx * 8 + i;
+    const int t = t0 + i;
     const bool in = t < p.n;
-    lse[i] = in ? p.lse[t] : 0.f;
+    lse[i] = in ? p.lse[t] * kLog2e : 0.f;
     g[i] = in ? p.g[t] : 0.f;
     y[i] = in ? p.targets[t] : -1;
   }
 #pragma unroll
-  for (int pass = 0; pass < 2; ++pass) {
-    const int vl = ty + pass * 32, v = v0 + vl;
-    u32x4 out = {0u, 0u, 0u, 0u};
-    if (v < p.V) {
-      uint16_t* src = p.zt + (int64_t)v * p.ld_z + t0 + tx * 8;
-      const u32x4 in = *(const u32x4*)src;
+  for (int step = 0; step < 8; ++step) {
+    const int v = v0 + step * 8 + ry;
+    if (v >= p.V) break;
+    uint16_t* ptr = p.zt + (int64_t)v * p.ld_z + t0;
+    const u32x4 in = *(const u32x4*)ptr;
+    u32x4 out;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const uint32_t w = in[i >> 1];
-        const float z = f16_bits_to_f32((uint16_t)((i & 1) ? (w >> 16) : (w & 0xffffu)));
-        float d = -__builtin_amdgcn_exp2f((z - lse[i]) * kLog2e);
-        if (v == y[i]) d += 1.f;
-        d *= g[i];
-        if (p.cap > 0.f) d *= 1.f - z * z * inv_cap2;
-        if (!(g[i] != 0.f)) d = 0.f;   // masked or padding token: exactly zero, whatever z holds
-        const uint32_t b = f32_to_bf16(d);
-        out[i >> 1] |= (i & 1) ? (b << 16) : b;
-      }
-      *(u32x4*)src = out;
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t w = in[i >> 1];
+      const float z = f16_bits_to_f32((uint16_t)((i & 1) ? (w >> 16) : (w & 0xffffu)));
+      float d = -__builtin_amdgcn_exp2f(fmaf(z, kLog2e, -lse[i]));
+      if (v == y[i]) d += 1.f;
+      d *= g[i];
+      if (p.cap > 0.f) d *= 1.f - z * z * inv_cap2;
+      if (!(g[i] != 0.f)) d = 0.f;   // masked or padding token: exactly zero, whatever z holds
+      const uint32_t b = f32_to_bf16(d);
+      if (i & 1) out[i >> 1] |= b << 16; else out[i >> 1] = b;
     }
-    *(u32x4*)&tile[vl][tx * 8] = out;
-  }
-  __syncthreads();
-  // transposed write: thread -> token tl, 8 consecutive vocab rows per 16-byte store
-#pragma unroll
-  for (int pass = 0; pass < 2; ++pass) {
-    const int tl = ty + pass * 32, t = t0 + tl;
-    const int vv = tx * 8;
-    if (t < p.n_pad && v0 + vv < p.V) {
-      u32x4 o;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        o[i] = (uint32_t)tile[vv + 2 * i][tl] | ((uint32_t)tile[vv + 2 * i + 1][tl] << 16);
-      *(u32x4*)(p.dz + (int64_t)t * p.ld_dz + v0 + vv) = o;
-    }
+    *(u32x4*)ptr = out;
   }
 }
 
 // ----------------------------------------------------------------------------- backward products
 struct DhArgs {
-  const __bf16* dz;   // [n, ld_dz]
+  const __bf16* dzt;  // [V, ld_z] dZ^T of the chunk
   const __bf16* w;    // [H, ld_w]
-  int64_t ld_dz, ld_w;
-  int n, H, V;
-  uint16_t* dh;       // chunk origin [n, ld_dh] bf16
+  int64_t ld_z, ld_w;
+  int n, n_pad, H, V;
+  int splits, k_per_split;   // vocab range of split s: [s*k_per_split, min(V, (s+1)*k_per_split))
+  uint16_t* dh;       // chunk origin [n, ld_dh] bf16 (splits == 1)
   int64_t ld_dh;
+  float* part;        // [splits, n_pad, H] fp32 partial sums (splits > 1)
 };
 
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap<4, 8> map) {
-  using G = GemmTN<BM, BN>;
+  using G = GemmTN<BM, BN, kKRow, kRowK>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int per = map.items();
+  const int split = blockIdx.x / per;
   int tm, tn;
-  if (!map.tile(blockIdx.x, tm, tn)) return;
+  if (!map.tile(blockIdx.x - split * per, tm, tn)) return;
   const int m0 = tm * BM, n0 = tn * BN;
+  const int k0 = split * p.k_per_split;
+  const int klen = min(p.V - k0, p.k_per_split);
   G g;
-  g.run(p.dz + (int64_t)m0 * p.ld_dz, p.n - m0, p.ld_dz, p.w + (int64_t)n0 * p.ld_w, p.H - n0, p.ld_w,
-        p.V, smem);
+  g.run(p.dzt + (int64_t)k0 * p.ld_z + m0, p.n_pad - m0, p.ld_z, p.w + (int64_t)n0 * p.ld_w + k0, p.H - n0,
+        p.ld_w, klen, smem);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
 #pragma unroll
@@ -346,77 +331,69 @@ __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap<4, 8> ma
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm * G::WM + mi * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
-        if (row < p.n) p.dh[(int64_t)row * p.ld_dh + col] = f32_to_bf16(g.acc[mi][ni][r]);
-      }
-  }
-}
-
-struct DwArgs {
-  const __bf16* ht;    // chunk origin inside hiddenT [H, ld_ht]
-  const __bf16* dzt;   // [V, ld_z]
-  int64_t ld_ht, ld_z;
-  int H, V, K;         // K = chunk tokens rounded up to 8 (padding holds zeros)
-  float* dw;           // [H, ld_w] f32
-  int64_t ld_dw;
-  int accumulate;
-};
-
-template <int BM, int BN>
-__global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap<4, 8> map) {
-  using G = GemmTN<BM, BN>;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  int tm, tn;
-  if (!map.tile(blockIdx.x, tm, tn)) return;
-  const int m0 = tm * BM, n0 = tn * BN;
-  G g;
-  g.run(p.ht + (int64_t)m0 * p.ld_ht, p.H - m0, p.ld_ht, p.dzt + (int64_t)n0 * p.ld_z, p.V - n0, p.ld_z,
-        p.K, smem);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
-#pragma unroll
-  for (int ni = 0; ni < G::NI; ++ni) {
-    const int col = n0 + wn * G::WN + ni * 32 + l31;
-    if (col >= p.V) continue;
-#pragma unroll
-    for (int mi = 0; mi < G::MI; ++mi)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * G::WM + mi * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
-        if (row < p.H) {
-          float* dst = p.dw + (int64_t)row * p.ld_dw + col;
-          *dst = p.accumulate ? *dst + g.acc[mi][ni][r] : g.acc[mi][ni][r];
+        if (row < p.n) {
+          if (p.splits == 1) p.dh[(int64_t)row * p.ld_dh + col] = f32_to_bf16(g.acc[mi][ni][r]);
+          else p.part[((int64_t)split * p.n_pad + row) * p.H + col] = g.acc[mi][ni][r];
         }
       }
   }
 }
 
-// ----------------------------------------------------------------------------- transpose
-// dst[c, r] = src[r, c] for r < R, c < C; dst columns R..R_pad-1 are zero-filled.
-// Requires C % 8 == 0, ld_dst % 8 == 0, R_pad % 8 == 0.  Block: 64 x 64 tile.
-__global__ __launch_bounds__(256) void k_transpose_bf16(const uint16_t* src, int64_t ld_src,
-                                                        uint16_t* dst, int64_t ld_dst, int R, int C,
-                                                        int R_pad) {
-  __shared__ uint16_t tile[64][72];
-  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
-  const int tx = threadIdx.x & 7, ty = threadIdx.x >> 3;
+// dh[row, :] = bf16(sum over splits of part[s, row, :]), fixed order.
+__global__ __launch_bounds__(256) void k_dhidden_reduce(const float* part, int splits, int n, int n_pad, int H,
+                                                        uint16_t* dh, int64_t ld_dh) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;   // one thread = 4 columns
+  const int h4 = H / 4;
+  if (i >= (int64_t)n * h4) return;
+  const int row = (int)(i / h4), c = (int)(i % h4) * 4;
+  f32x4 a = *(const f32x4*)(part + (int64_t)row * H + c);
+  for (int s = 1; s < splits; ++s) a += *(const f32x4*)(part + ((int64_t)s * n_pad + row) * H + c);
+  uint16_t* o = dh + (int64_t)row * ld_dh + c;
+  const uint32_t lo = f32_to_bf16(a[0]) | ((uint32_t)f32_to_bf16(a[1]) << 16);
+  const uint32_t hi = f32_to_bf16(a[2]) | ((uint32_t)f32_to_bf16(a[3]) << 16);
+  *(uint2*)o = make_uint2(lo, hi);
+}
+
+struct DwArgs {
+  const __bf16* dzt;   // [V, ld_z] dZ^T of the chunk
+  const __bf16* hid;   // chunk origin [n, ld_hid]
+  int64_t ld_z, ld_hid;
+  int H, V, n;         // n = tokens of the chunk (dZ^T holds zeros from n up to its padded width)
+  float* dw;           // [H, ld_dw] f32
+  int64_t ld_dw;
+  int accumulate;
+};
+
+// Tile of dW^T: rows = vocab (MFMA row direction), columns = hidden (lanes).  A lane's four
+// consecutive accumulator rows are four consecutive floats of one dW row: 16-byte accesses.
+template <int BM, int BN>
+__global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap<4, 8> map) {
+  using G = GemmTN<BM, BN, kRowK, kKRow>;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  int tm, tn;
+  if (!map.tile(blockIdx.x, tm, tn)) return;
+  const int m0 = tm * BM, n0 = tn * BN;
+  G g;
+  g.run(p.dzt + (int64_t)m0 * p.ld_z, p.V - m0, p.ld_z, p.hid + n0, p.H - n0, p.ld_hid, p.n, smem);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
 #pragma unroll
-  for (int pass = 0; pass < 2; ++pass) {
-    const int rl = ty + pass * 32, r = r0 + rl, c = c0 + tx * 8;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (r < R && c < C) v = *(const u32x4*)(src + (int64_t)r * ld_src + c);
-    *(u32x4*)&tile[rl][tx * 8] = v;
-  }
-  __syncthreads();
+  for (int ni = 0; ni < G::NI; ++ni) {
+    const int h = n0 + wn * G::WN + ni * 32 + l31;
+    if (h >= p.H) continue;
+    float* row = p.dw + (int64_t)h * p.ld_dw;
 #pragma unroll
-  for (int pass = 0; pass < 2; ++pass) {
-    const int cl = ty + pass * 32, c = c0 + cl, r = r0 + tx * 8;
-    if (c < C && r < R_pad) {
-      u32x4 o;
+    for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        o[i] = (uint32_t)tile[tx * 8 + 2 * i][cl] | ((uint32_t)tile[tx * 8 + 2 * i + 1][cl] << 16);
-      *(u32x4*)(dst + (int64_t)c * ld_dst + r) = o;
-    }
+      for (int q = 0; q < 4; ++q) {
+        const int v = m0 + wm * G::WM + mi * 32 + q * 8 + lhi * 4;
+        if (v < p.V) {   // V % 8 == 0: the four columns are in or out together
+          f32x4 a = {g.acc[mi][ni][q * 4], g.acc[mi][ni][q * 4 + 1], g.acc[mi][ni][q * 4 + 2],
+                     g.acc[mi][ni][q * 4 + 3]};
+          if (p.accumulate) a += *(const f32x4*)(row + v);
+          *(f32x4*)(row + v) = a;
+        }
+      }
   }
 }
 
