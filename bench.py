@@ -34,6 +34,9 @@ def main() -> int:
     ap.add_argument("--chunk-tokens", type=int, default=0)
     ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB (a kernel of known traffic, to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the loss path on ONE GPU (no collectives, no sharding); "
@@ -69,6 +72,12 @@ def main() -> int:
             total_valid_token_count=wl["total_valid_token_count"], seq_shape=wl["seq_shape"],
             return_token_entropy=cfg.token_entropy, **kw)
 
+    if args.copy_calibration_mib:
+        src = torch.empty(args.copy_calibration_mib << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

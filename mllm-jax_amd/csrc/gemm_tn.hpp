@@ -55,20 +55,22 @@ MJ_DEV void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc07f); }
 
 // Maps a linear workgroup id to a tile so that (a) the 32 workgroups that land on one
 // XCD at a time (ids congruent mod 8 go to the same XCD) form a GM x GN block of tiles
-// sharing operand slices in that XCD's L2, and (b) consecutive blocks walk along M first.
+// sharing operand slices in that XCD's L2, and (b) consecutive blocks -- the ones the eight
+// XCDs work on at the same time -- walk along N first (n_first) or along M first.
 template <int GM, int GN>
 struct TileMap {
-  int tiles_m, tiles_n, sb_m, sb_n;
-  __host__ __device__ TileMap(int tm, int tn)
-      : tiles_m(tm), tiles_n(tn), sb_m((tm + GM - 1) / GM), sb_n((tn + GN - 1) / GN) {}
+  int tiles_m, tiles_n, sb_m, sb_n, n_first;
+  __host__ __device__ TileMap(int tm, int tn, int n_first_ = 0)
+      : tiles_m(tm), tiles_n(tn), sb_m((tm + GM - 1) / GM), sb_n((tn + GN - 1) / GN), n_first(n_first_) {}
   __host__ __device__ int items() const { return ((sb_m * sb_n + 7) / 8) * 8 * (GM * GN); }
   __host__ int grid() const { return items(); }
   MJ_DEV bool tile(int pid, int& tm, int& tn) const {
     const int xcd = pid & 7, q = pid >> 3;
     const int sb = (q / (GM * GN)) * 8 + xcd, within = q % (GM * GN);
     if (sb >= sb_m * sb_n) return false;
-    tm = (sb % sb_m) * GM + within % GM;
-    tn = (sb / sb_m) * GN + within / GM;
+    const int bm = n_first ? sb / sb_n : sb % sb_m, bn = n_first ? sb % sb_n : sb / sb_m;
+    tm = bm * GM + within % GM;
+    tn = bn * GN + within / GM;
     return tm < tiles_m && tn < tiles_n;
   }
 };

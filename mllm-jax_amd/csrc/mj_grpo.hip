@@ -185,7 +185,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       a.zt = bwd ? zt : nullptr; a.ld_z = p.n_pad;
       a.pm = pm; a.pl = pl; a.ps = ps; a.ld_p = p.n_pad;
       a.targets = targets + c0; a.zy = zy + c0;
-      mj::TileMap<4, 8> map((V + BM - 1) / BM, (nc + BN - 1) / BN);
+      mj::TileMap<4, 8> map((V + BM - 1) / BM, (nc + BN - 1) / BN, 1);
       Timed t(MJ_GRPO_K_LOGITS_STATS, st);
       mj::k_logits_stats<BM, BN><<<map.grid(), mj::kThreads, lds, st>>>(a, map);
     }
@@ -225,7 +225,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       h.splits = p.dh_splits; h.k_per_split = (int)p.dh_k_per_split;
       h.dh = (uint16_t*)d_hidden + c0 * d->ld_hidden; h.ld_dh = d->ld_hidden;
       h.part = part;
-      mj::TileMap<4, 8> mh((nc + BM - 1) / BM, (H + BN - 1) / BN);
+      mj::TileMap<4, 8> mh((nc + BM - 1) / BM, (H + BN - 1) / BN, 0);
       {
         Timed t(MJ_GRPO_K_DHIDDEN, st);
         mj::k_dhidden<BM, BN><<<mh.grid() * h.splits, mj::kThreads, lds, st>>>(h, mh);
@@ -242,7 +242,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       w.H = H; w.V = V; w.n = nc;
       w.dw = d_w; w.ld_dw = d->ld_w;
       w.accumulate = (c0 > 0 || (d->flags & MJ_GRPO_FLAG_DW_ACCUMULATE)) ? 1 : 0;
-      mj::TileMap<4, 8> mw((V + BM - 1) / BM, (H + BN - 1) / BN);
+      mj::TileMap<4, 8> mw((V + BM - 1) / BM, (H + BN - 1) / BN, 0);
       {
         Timed t(MJ_GRPO_K_DW, st);
         mj::k_dw<BM, BN><<<mw.grid(), mj::kThreads, lds, st>>>(w, mw);
