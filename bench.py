@@ -20,9 +20,15 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (profiles/), keyed by (config index, kernel); None until measured for that workload.
-MEASURED_TRAFFIC_BYTES = {}
+# Bytes per launch that crossed the L2 <-> fabric boundary (Infinity Cache or HBM behind it), from
+# two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for
+# a plain 1 GiB device copy (x2.00 fetch, x1.00 write); summary in profiles/.  Keyed by
+# (config index, kernel); None for workloads that were not counted.
+MEASURED_TRAFFIC_BYTES = {
+    (2, "k_logits_stats"): 16.78e9,
+    (2, "k_dhidden"): 21.80e9,
+    (2, "k_dw"): 17.41e9,
+}
 
 
 def main() -> int:
@@ -32,7 +38,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (default 2)")
     ap.add_argument("--chunk-tokens", type=int, default=0)
-    ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known traffic, to scale "
