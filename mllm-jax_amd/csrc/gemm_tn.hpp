@@ -1,7 +1,7 @@
 // gemm_tn.hpp -- bf16 MFMA tile engine for gfx950 (CDNA4), wave64.
 //
-// C[M,N] (fp32 accumulators) = sum_k A(m,k) * B(n,k).  One workgroup of 256 threads
-// (4 wavefronts, 2x2) owns a BM x BN tile; each wavefront owns (BM/2) x (BN/2) as a grid of
+// C[M,N] (fp32 accumulators) = sum_k A(m,k) * B(n,k).  One workgroup of WAVES_M x WAVES_N
+// wavefronts owns a BM x BN tile; each wavefront owns (BM/WAVES_M) x (BN/WAVES_N) as a grid of
 // 32x32 MFMA blocks (v_mfma_f32_32x32x16_bf16).
 //
 // Each operand may live in memory in either of two layouts, so no operand ever needs a
@@ -76,10 +76,12 @@ struct TileMap {
 };
 
 // One operand of the tile: ROWS tile rows (M or N direction) by 64 k per slice, 128*ROWS bytes of
-// LDS per stage, ROWS/32 16-byte chunks per thread per slice.
-template <int ROWS, int LAYOUT>
+// LDS per stage, ROWS*8/THREADS 16-byte chunks per thread per slice.
+template <int ROWS, int LAYOUT, int THREADS>
 struct Operand {
-  static constexpr int LD = ROWS / 32;
+  static constexpr int LD = ROWS * 8 / THREADS;
+  static constexpr int RPP = THREADS / 8;          // kRowK: tile rows covered by one pass of the workgroup
+  static constexpr int KPP = THREADS / (ROWS / 8); // kKRow: k-rows covered by one pass
   static constexpr int kBytes = ROWS * 128;
 
   const char* base;      // tile origin: (row 0, k 0)
@@ -97,7 +99,7 @@ struct Operand {
   // ({r..r+3} and {r+8..r+11}) must land in 8 different segments of the 512-byte row.
   static MJ_DEV int sigma(int krow) { return (krow & 3) | ((krow >> 1) & 4); }
   // 16-byte chunk permutation of the kRowK image (see the file header).
-  static MJ_DEV int swz(int r) { return (r ^ (r >> 3)) & 7; }
+  static MJ_DEV int swz(int r) { return (r & 7) ^ ((r >> 3) & 3); }   // depends on r mod 32 only
 
   MJ_DEV void init(const __bf16* p, int rows_valid, int64_t ld, int K_, int wave_row0) {
     static_assert(LAYOUT == kRowK || ROWS == 256, "the k-major image is laid out for 256-row tiles");
@@ -107,12 +109,12 @@ struct Operand {
     rows = rows_valid < ROWS ? rows_valid : ROWS;
     K = K_;
     if (LAYOUT == kRowK) {
-      const int row = t >> 3, chunk = t & 7;     // chunk t%8 of tile rows t/8 + 32*i
+      const int row = t >> 3, chunk = t & 7;     // chunk t%8 of tile rows t/8 + RPP*i
       rsrc = make_rsrc(base, (int64_t)rows * ld2);
 #pragma unroll
-      for (int i = 0; i < LD; ++i) goff[i] = (uint32_t)((row + 32 * i) * ld2 + chunk * 16);
+      for (int i = 0; i < LD; ++i) goff[i] = (uint32_t)((row + RPP * i) * ld2 + chunk * 16);
       klimit = K - chunk * 8;
-      st_off = row * 128 + ((chunk ^ swz(row)) << 4);   // swz(row + 32*i) == swz(row)
+      st_off = row * 128 + ((chunk ^ swz(row)) << 4);   // swz(row + RPP*i) == swz(row)
       st_off1 = st_off;
       col_ok = true;
       const int l31 = lane & 31, lhi = lane >> 5;       // fragment row, k-chunk 2*ks + lane/32
@@ -121,13 +123,13 @@ struct Operand {
         rd[ks] = (wave_row0 + l31) * 128 + (((2 * ks + lhi) ^ swz(l31)) << 4);
     } else {
       constexpr int CPR = ROWS / 8;              // 16-byte chunks per k-row
-      const int krow = t / CPR, chunk = t % CPR; // chunk of k-rows krow + 8*i
+      const int krow = t / CPR, chunk = t % CPR; // chunk of k-rows krow + KPP*i
 #pragma unroll
-      for (int i = 0; i < LD; ++i) goff[i] = (uint32_t)((krow + (256 / CPR) * i) * ld2 + chunk * 16);
+      for (int i = 0; i < LD; ++i) goff[i] = (uint32_t)((krow + KPP * i) * ld2 + chunk * 16);
       col_ok = chunk * 8 < rows;
       klimit = 0;
       st_off = krow * (ROWS * 2) + ((chunk ^ (sigma(krow) << 2)) << 4);
-      st_off1 = krow * (ROWS * 2) + ((chunk ^ (sigma(krow + 8) << 2)) << 4);
+      st_off1 = krow * (ROWS * 2) + ((chunk ^ (sigma(krow + KPP) << 2)) << 4);   // differs only if KPP == 8
       // Transposing read: the 16 lanes of a group fetch 4 k-rows x 4 row-quads (8 bytes each) and
       // get back, lane i, the 4 k of row i.  Lane l: group g = l/16, s = l%16 reads k-row
       // (g/2)*8 + s/4 (+4 for the second read, +16*ks), quad (g%2)*4 + s%4 of the 32-row fragment.
@@ -158,9 +160,9 @@ struct Operand {
   }
   MJ_DEV void store(char* stage, int i, u32x4 v) const {
     if (LAYOUT == kRowK)
-      *(u32x4*)(stage + st_off + i * 32 * 128) = v;
+      *(u32x4*)(stage + st_off + i * RPP * 128) = v;
     else
-      *(u32x4*)(stage + ((i & 1) ? st_off1 : st_off) + i * 8 * (ROWS * 2)) = v;
+      *(u32x4*)(stage + ((i & 1) ? st_off1 : st_off) + i * KPP * (ROWS * 2)) = v;
   }
   // MFMA fragment f (32 rows) of k-step ks.
   MJ_DEV bf16x8 frag(const char* stage, int f, int ks) const {
@@ -174,13 +176,15 @@ struct Operand {
   }
 };
 
-template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK>
+template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK, int WAVES_M = 2, int WAVES_N = 2>
 struct GemmTN {
   static_assert(BM % 32 == 0 && BN % 32 == 0, "tile sides are multiples of 32");
-  static constexpr int WM = BM / 2, WN = BN / 2;     // wavefront tile
+  static constexpr int kWavesM = WAVES_M, kWavesN = WAVES_N;
+  static constexpr int kThreads = 64 * WAVES_M * WAVES_N;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;   // wavefront tile
   static constexpr int MI = WM / 32, NI = WN / 32;   // 32x32 blocks per wavefront
-  using OpA = Operand<BM, LAY_A>;
-  using OpB = Operand<BN, LAY_B>;
+  using OpA = Operand<BM, LAY_A, kThreads>;
+  using OpB = Operand<BN, LAY_B, kThreads>;
   static constexpr int A_LD = OpA::LD, B_LD = OpB::LD;
   static constexpr int LPS = A_LD + B_LD;            // 16-byte chunks per thread per slice
   static constexpr int kStageBytes = OpA::kBytes + OpB::kBytes;
@@ -196,7 +200,7 @@ struct GemmTN {
   MJ_DEV void run(const __bf16* A, int rows_a, int64_t lda, const __bf16* B, int rows_b,
                   int64_t ldb, int K, char* smem) {
     const int wave = threadIdx.x >> 6;
-    const int wm = wave & 1, wn = wave >> 1;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     OpA a;
     OpB b;
     a.init(A, rows_a, lda, K, wm * WM);

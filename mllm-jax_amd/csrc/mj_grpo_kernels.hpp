@@ -42,6 +42,22 @@ MJ_DEV float softcap_apply(float z, float cap, float inv_cap) {
   return cap * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e));
 }
 
+// Epilogue stores go through buffer descriptors: the row part of the address is a scalar offset,
+// the lane part is computed once, and rows past the end of the output fall outside the
+// descriptor's range and are dropped -- no per-store address arithmetic or branches.
+MJ_DEV void store_b16(uint16_t v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  __builtin_amdgcn_raw_buffer_store_b16((short)v, r, voff, soff, 0);
+}
+MJ_DEV void store_b32(float v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, voff, soff, 0);
+}
+MJ_DEV void store_b128(f32x4 v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff, soff, 0);
+}
+MJ_DEV f32x4 load_b128(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+
 // ----------------------------------------------------------------------------- logits + stats
 struct LogitsArgs {
   const __bf16* w;       // lm_head [H, ld_w]
@@ -73,6 +89,10 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
   const int vbase = vwave + lhi * 4;             // + mi*32 + (r/4)*8 + r%4
   const bool tail = (m0 + BM > p.V);
   const float inv_cap = p.cap > 0.f ? 1.f / p.cap : 0.f;
+  // this wavefront's 128 rows of logits^T; rows at or past V fall outside and are dropped
+  const uint32_t ldz2 = (uint32_t)p.ld_z * 2;
+  const int zrows = min(max(p.V - vwave, 0), G::WM);
+  const __amdgpu_buffer_rsrc_t zrs = make_rsrc(p.zt + (int64_t)vwave * p.ld_z, (int64_t)zrows * ldz2);
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
     const int col = n0 + wn * G::WN + ni * 32 + l31;
@@ -125,13 +145,12 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
       }
     }
     if (p.zt != nullptr) {
+      const uint32_t voff = (uint32_t)((lhi * 4 * p.ld_z + col) * 2);
 #pragma unroll
       for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int v = vbase + mi * 32 + (r >> 2) * 8 + (r & 3);
-          if (!tail || v < p.V) p.zt[(int64_t)v * p.ld_z + col] = f32_to_f16_bits(g.acc[mi][ni][r]);
-        }
+        for (int r = 0; r < 16; ++r)
+          store_b16(f32_to_f16_bits(g.acc[mi][ni][r]), zrs, voff, (uint32_t)(mi * 32 + (r >> 2) * 8 + (r & 3)) * ldz2);
     }
   }
 }
@@ -322,20 +341,35 @@ __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap<4, 8> ma
         p.ld_w, klen, smem);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
+  const int row0 = m0 + wm * G::WM;                       // first token row of this wavefront
+  const int rows = min(max(p.n - row0, 0), G::WM);        // rows at or past n are dropped
+  if (p.splits == 1) {
+    const uint32_t ld2 = (uint32_t)p.ld_dh * 2;
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.dh + (int64_t)row0 * p.ld_dh, (int64_t)rows * ld2);
 #pragma unroll
-  for (int ni = 0; ni < G::NI; ++ni) {
-    const int col = n0 + wn * G::WN + ni * 32 + l31;
-    if (col >= p.H) continue;
+    for (int ni = 0; ni < G::NI; ++ni) {
+      const int col = n0 + wn * G::WN + ni * 32 + l31;
+      const uint32_t voff = col < p.H ? (uint32_t)(lhi * 4 * ld2 + col * 2) : kOob;
 #pragma unroll
-    for (int mi = 0; mi < G::MI; ++mi)
+      for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * G::WM + mi * 32 + (r >> 2) * 8 + lhi * 4 + (r & 3);
-        if (row < p.n) {
-          if (p.splits == 1) p.dh[(int64_t)row * p.ld_dh + col] = f32_to_bf16(g.acc[mi][ni][r]);
-          else p.part[((int64_t)split * p.n_pad + row) * p.H + col] = g.acc[mi][ni][r];
-        }
-      }
+        for (int r = 0; r < 16; ++r)
+          store_b16(f32_to_bf16(g.acc[mi][ni][r]), rs, voff, (uint32_t)(mi * 32 + (r >> 2) * 8 + (r & 3)) * ld2);
+    }
+  } else {
+    const uint32_t ld4 = (uint32_t)p.H * 4;
+    const __amdgpu_buffer_rsrc_t rs =
+        make_rsrc(p.part + ((int64_t)split * p.n_pad + row0) * p.H, (int64_t)rows * ld4);
+#pragma unroll
+    for (int ni = 0; ni < G::NI; ++ni) {
+      const int col = n0 + wn * G::WN + ni * 32 + l31;
+      const uint32_t voff = col < p.H ? (uint32_t)(lhi * 4 * ld4 + col * 4) : kOob;
+#pragma unroll
+      for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          store_b32(g.acc[mi][ni][r], rs, voff, (uint32_t)(mi * 32 + (r >> 2) * 8 + (r & 3)) * ld4);
+    }
   }
 }
 
@@ -377,22 +411,26 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap<4, 8> map) {
   g.run(p.dzt + (int64_t)m0 * p.ld_z, p.V - m0, p.ld_z, p.hid + n0, p.H - n0, p.ld_hid, p.n, smem);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
+  // dW rows of this wavefront's 128 hidden columns, starting at its first vocab column; a lane's
+  // address is (its hidden row) * ld + (its 4-float group), the vocab block is the scalar offset.
+  const int h0 = n0 + wn * G::WN, v0 = m0 + wm * G::WM;
+  const int hrows = min(max(p.H - h0, 0), G::WN);
+  const uint32_t ld4 = (uint32_t)p.ld_dw * 4;
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.dw + (int64_t)h0 * p.ld_dw + v0, (int64_t)hrows * ld4 - (int64_t)v0 * 4);
+  const int vleft = p.V - v0;                            // V % 8 == 0: groups of 4 are in or out together
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
-    const int h = n0 + wn * G::WN + ni * 32 + l31;
-    if (h >= p.H) continue;
-    float* row = p.dw + (int64_t)h * p.ld_dw;
+    const uint32_t lane_off = (uint32_t)((ni * 32 + l31) * ld4 + lhi * 16);
 #pragma unroll
     for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int v = m0 + wm * G::WM + mi * 32 + q * 8 + lhi * 4;
-        if (v < p.V) {   // V % 8 == 0: the four columns are in or out together
-          f32x4 a = {g.acc[mi][ni][q * 4], g.acc[mi][ni][q * 4 + 1], g.acc[mi][ni][q * 4 + 2],
-                     g.acc[mi][ni][q * 4 + 3]};
-          if (p.accumulate) a += *(const f32x4*)(row + v);
-          *(f32x4*)(row + v) = a;
-        }
+        const int vv = mi * 32 + q * 8;
+        const uint32_t voff = (vv + lhi * 4) < vleft ? lane_off : kOob;
+        f32x4 a = {g.acc[mi][ni][q * 4], g.acc[mi][ni][q * 4 + 1], g.acc[mi][ni][q * 4 + 2],
+                   g.acc[mi][ni][q * 4 + 3]};
+        if (p.accumulate) a += load_b128(rs, voff, (uint32_t)vv * 4);
+        store_b128(a, rs, voff, (uint32_t)vv * 4);
       }
   }
 }
