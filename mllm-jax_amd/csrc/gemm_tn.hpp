@@ -50,6 +50,17 @@ MJ_DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int64_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)capped, 0x00020000);
 }
 
+// Same, for descriptors built from per-wavefront (not per-workgroup) quantities: the pieces are
+// pinned to scalar registers so that the memory instructions need no per-lane descriptor loop.
+MJ_DEV __amdgpu_buffer_rsrc_t make_rsrc_wave(const void* p, int64_t bytes) {
+  const uint64_t a = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  const int64_t capped = bytes < 0 ? 0 : (bytes > 0x7fffff00 ? 0x7fffff00 : bytes);
+  const int n = __builtin_amdgcn_readfirstlane((int)capped);
+  return __builtin_amdgcn_make_buffer_rsrc((void*)(((uint64_t)hi << 32) | lo), 0, n, 0x00020000);
+}
+
 // s_waitcnt with only the LDS/scalar counter constrained (gfx9 encoding).
 MJ_DEV void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc07f); }
 

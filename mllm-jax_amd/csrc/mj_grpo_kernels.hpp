@@ -83,7 +83,8 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
   G g;
   g.run(p.w + m0, p.V - m0, p.ld_w, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0, p.ld_hid, p.H, smem);
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps descriptors in SGPRs
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
   const int vwave = m0 + wm * G::WM;             // first vocab row of this wavefront
   const int vbase = vwave + lhi * 4;             // + mi*32 + (r/4)*8 + r%4
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
   // this wavefront's 128 rows of logits^T; rows at or past V fall outside and are dropped
   const uint32_t ldz2 = (uint32_t)p.ld_z * 2;
   const int zrows = min(max(p.V - vwave, 0), G::WM);
-  const __amdgpu_buffer_rsrc_t zrs = make_rsrc(p.zt + (int64_t)vwave * p.ld_z, (int64_t)zrows * ldz2);
+  const __amdgpu_buffer_rsrc_t zrs = make_rsrc_wave(p.zt + (int64_t)vwave * p.ld_z, (int64_t)zrows * ldz2);
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
     const int col = n0 + wn * G::WN + ni * 32 + l31;
@@ -339,13 +340,14 @@ __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap<4, 8> ma
   G g;
   g.run(p.dzt + (int64_t)k0 * p.ld_z + m0, p.n_pad - m0, p.ld_z, p.w + (int64_t)n0 * p.ld_w + k0, p.H - n0,
         p.ld_w, klen, smem);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps descriptors in SGPRs
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
   const int row0 = m0 + wm * G::WM;                       // first token row of this wavefront
   const int rows = min(max(p.n - row0, 0), G::WM);        // rows at or past n are dropped
   if (p.splits == 1) {
     const uint32_t ld2 = (uint32_t)p.ld_dh * 2;
-    const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.dh + (int64_t)row0 * p.ld_dh, (int64_t)rows * ld2);
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc_wave(p.dh + (int64_t)row0 * p.ld_dh, (int64_t)rows * ld2);
 #pragma unroll
     for (int ni = 0; ni < G::NI; ++ni) {
       const int col = n0 + wn * G::WN + ni * 32 + l31;
@@ -359,7 +361,7 @@ __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap<4, 8> ma
   } else {
     const uint32_t ld4 = (uint32_t)p.H * 4;
     const __amdgpu_buffer_rsrc_t rs =
-        make_rsrc(p.part + ((int64_t)split * p.n_pad + row0) * p.H, (int64_t)rows * ld4);
+        make_rsrc_wave(p.part + ((int64_t)split * p.n_pad + row0) * p.H, (int64_t)rows * ld4);
 #pragma unroll
     for (int ni = 0; ni < G::NI; ++ni) {
       const int col = n0 + wn * G::WN + ni * 32 + l31;
@@ -409,14 +411,15 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap<4, 8> map) {
   const int m0 = tm * BM, n0 = tn * BN;
   G g;
   g.run(p.dzt + (int64_t)m0 * p.ld_z, p.V - m0, p.ld_z, p.hid + n0, p.H - n0, p.ld_hid, p.n, smem);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps descriptors in SGPRs
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
   // dW rows of this wavefront's 128 hidden columns, starting at its first vocab column; a lane's
   // address is (its hidden row) * ld + (its 4-float group), the vocab block is the scalar offset.
   const int h0 = n0 + wn * G::WN, v0 = m0 + wm * G::WM;
   const int hrows = min(max(p.H - h0, 0), G::WN);
   const uint32_t ld4 = (uint32_t)p.ld_dw * 4;
-  const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.dw + (int64_t)h0 * p.ld_dw + v0, (int64_t)hrows * ld4 - (int64_t)v0 * 4);
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc_wave(p.dw + (int64_t)h0 * p.ld_dw + v0, (int64_t)hrows * ld4 - (int64_t)v0 * 4);
   const int vleft = p.V - v0;                            // V % 8 == 0: groups of 4 are in or out together
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
