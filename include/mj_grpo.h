@@ -63,6 +63,9 @@ typedef struct MjGrpoDesc {
   float grad_loss_scale; /* upstream d(loss); 1 for a terminal loss */
   uint32_t flags;
   uint32_t reserved;
+  float entropy_coef;    /* PPOActorCriticModule.entropy_coef (plugins/training/ppo/module.py:140):
+                            the loss becomes policy_loss - entropy_coef * entropy; 0 = GRPO */
+  float inv_entropy_count; /* 1 / (sum(mask) + 1e-8), the normaliser of that entropy (:79); 0 = unused */
 } MjGrpoDesc;
 
 /* Library version, MAJOR*10000 + MINOR*100 + PATCH. */
@@ -79,7 +82,9 @@ int mj_grpo_workspace_bytes(const MjGrpoDesc* desc, size_t* forward_bytes,
  * gather), :136-138 (per-token entropy), :161-180 (ratio, clip, min, masked normalised sum)
  * on top of the lm_head product (qwen2/modular_qwen2.py:182), streaming over vocab tiles:
  * no [N,V] tensor is written.  Outputs: logp[N], lse[N], token_entropy[N] (may be NULL),
- * loss[1].  */
+ * loss[2]: loss[0] = policy loss - entropy_coef * entropy, loss[1] = entropy =
+ * sum(token_entropy * mask) * inv_entropy_count (plugins/training/ppo/module.py:77-79; 0 when
+ * inv_entropy_count is 0).  */
 int mj_grpo_forward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
                     const int32_t* targets, const float* old_logp, const float* advantages,
                     const float* mask, float* logp, float* lse, float* token_entropy,
@@ -89,7 +94,9 @@ int mj_grpo_forward(const MjGrpoDesc* desc, const void* hidden, const void* lm_h
  * jax.value_and_grad(loss_fn) of plugins/training/update/train_step.py:15-24 restricted to
  * the lm_head + loss part: besides the forward outputs it writes
  * d_hidden[N, ld_hidden] bf16 and d_lm_head[H, ld_w] f32, both already multiplied by
- * grad_loss_scale.  The workspace holds 16-bit (half) logits for chunk_tokens tokens at a time. */
+ * grad_loss_scale.  The workspace holds 16-bit (half) logits for chunk_tokens tokens at a time.
+ * With entropy_coef != 0 the gradient includes the entropy bonus,
+ * d(-coef*entropy)/dz = coef * mask * inv_entropy_count * p * (log p + H_t). */
 int mj_grpo_forward_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
                              const int32_t* targets, const float* old_logp,
                              const float* advantages, const float* mask, float* logp,
@@ -100,7 +107,7 @@ int mj_grpo_forward_backward(const MjGrpoDesc* desc, const void* hidden, const v
 /* Backward from a saved forward (lse[N], logp[N]): recomputes the logits chunk by chunk
  * (8*N*H*V flop with the forward).  Same outputs as the backward half above.  For callers
  * that must separate the two passes (e.g. a forward under no-grad followed later by a
- * backward with a non-unit upstream gradient). */
+ * backward with a non-unit upstream gradient).  entropy_coef must be 0 here. */
 int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
                      const int32_t* targets, const float* old_logp, const float* advantages,
                      const float* mask, const float* lse, const float* logp, void* d_hidden,

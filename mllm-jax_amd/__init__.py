@@ -1,8 +1,8 @@
 """MI355X-native fused GRPO loss (lm_head product + streaming log-softmax + clipped
 policy-ratio loss, forward and backward) behind the reference's loss-function contract."""
-from .loss import (TrainGRPOModule, grpo_fused_loss, grpo_loss_value_and_grad, loss_and_metrics,
+from .loss import (PPOActorCriticModule, TrainGRPOModule, grpo_fused_loss, grpo_loss_value_and_grad, loss_and_metrics,
                    release_workspaces, sft_fused_loss)
 from .workloads import CONFIGS, LossConfig, make_workload
 
-__all__ = ["TrainGRPOModule", "grpo_fused_loss", "grpo_loss_value_and_grad", "loss_and_metrics",
+__all__ = ["TrainGRPOModule", "PPOActorCriticModule", "grpo_fused_loss", "grpo_loss_value_and_grad", "loss_and_metrics",
            "sft_fused_loss", "release_workspaces", "CONFIGS", "LossConfig", "make_workload"]

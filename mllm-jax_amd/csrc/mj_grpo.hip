@@ -55,7 +55,7 @@ struct Plan {
   int dh_splits;          // vocab splits of the dHidden product (1 = none)
   int64_t dh_k_per_split;
   // byte offsets into the workspace
-  size_t zy, term, pm, pl, ps, g, zt, part, total_fwd, total_bwd;
+  size_t zy, term, eterm, pm, pl, ps, g, ge, hent, zt, part, total_fwd, total_bwd;
 };
 
 // Splits of the dHidden product over the vocab: its (n/256) x (H/256) tiles rarely fill the 256
@@ -88,6 +88,8 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   if (d->softcap < 0.f || !isfinite(d->softcap)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "softcap must be >= 0");
   if (d->chunk_tokens < 0) return fail(MJ_GRPO_ERR_SHAPE, "chunk_tokens must be >= 0");
   if (!isfinite(d->inv_total_valid_tokens)) return fail(MJ_GRPO_ERR_SHAPE, "inv_total_valid_tokens not finite");
+  if (!isfinite(d->entropy_coef) || !isfinite(d->inv_entropy_count) || d->inv_entropy_count < 0.f)
+    return fail(MJ_GRPO_ERR_SHAPE, "entropy_coef / inv_entropy_count not finite");
   p->N = d->n_tokens; p->H = d->hidden; p->V = d->vocab;
   int64_t chunk = d->chunk_tokens > 0 ? d->chunk_tokens : kDefaultChunk;
   chunk = rup(chunk, 256);
@@ -101,10 +103,13 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   auto take = [&](size_t bytes) { size_t at = o; o = (size_t)rup((int64_t)(o + bytes), 256); return at; };
   p->zy = take((size_t)p->N * 4);
   p->term = take((size_t)p->N * 4);
+  p->eterm = take((size_t)p->N * 4);
   p->pm = take((size_t)p->parts * p->n_pad * 4);
   p->pl = take((size_t)p->parts * p->n_pad * 4);
   p->ps = take((size_t)p->parts * p->n_pad * 4);
   p->g = take((size_t)p->n_pad * 4);
+  p->ge = take((size_t)p->n_pad * 4);
+  p->hent = take((size_t)p->n_pad * 4);
   p->total_fwd = o;
   p->zt = take((size_t)p->V * p->n_pad * 2);
   p->part = take(p->dh_splits > 1 ? (size_t)p->dh_splits * p->n_pad * p->H * 4 : 0);
@@ -146,6 +151,8 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
   if (!sft && !adv) return fail(MJ_GRPO_ERR_NULL, "advantages is NULL");
   if (mode != kBackwardOnly && (!logp || !lse || !loss)) return fail(MJ_GRPO_ERR_NULL, "logp/lse/loss output is NULL");
   if (mode == kBackwardOnly && (!saved_lse || !saved_logp)) return fail(MJ_GRPO_ERR_NULL, "saved lse/logp is NULL");
+  if (mode == kBackwardOnly && d->entropy_coef != 0.f)
+    return fail(MJ_GRPO_ERR_UNSUPPORTED, "the separate backward does not carry the entropy bonus (entropy_coef must be 0)");
   if (bwd && (!d_hidden || !d_w)) return fail(MJ_GRPO_ERR_NULL, "d_hidden/d_lm_head is NULL");
   if (!workspace) return fail(MJ_GRPO_ERR_WORKSPACE, "workspace is NULL");
   const size_t need = bwd ? p.total_bwd : p.total_fwd;
@@ -159,6 +166,10 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
   const int N = (int)p.N, H = (int)p.H, V = (int)p.V;
   float* zy = (float*)(ws + p.zy);
   float* term = (float*)(ws + p.term);
+  float* eterm = (float*)(ws + p.eterm);
+  float* ge = (float*)(ws + p.ge);
+  float* hent = (float*)(ws + p.hent);
+  const bool bonus = bwd && d->entropy_coef != 0.f;
   float* pm = (float*)(ws + p.pm);
   float* pl = (float*)(ws + p.pl);
   float* ps = (float*)(ws + p.ps);
@@ -199,6 +210,8 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       f.gscale = gscale; f.sft = sft ? 1 : 0;
       f.logp = logp + c0; f.lse = lse + c0; f.ent = ent ? ent + c0 : nullptr;
       f.term = term + c0; f.g = bwd ? g : nullptr;
+      f.ent_coef = d->entropy_coef; f.inv_ent_cnt = d->inv_entropy_count; f.eterm = eterm + c0;
+      f.ge = bonus ? ge : nullptr; f.hent = bonus ? hent : nullptr;
       Timed t(MJ_GRPO_K_FINALIZE, st);
       mj::k_finalize<<<n_pad / 64, 256, 0, st>>>(f);
     } else {
@@ -211,6 +224,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       mj::DzArgs z;
       z.zt = zt; z.ld_z = p.n_pad;
       z.lse = (mode == kBackwardOnly ? saved_lse : lse) + c0; z.g = g; z.targets = targets + c0;
+      z.ge = bonus ? ge : nullptr; z.hent = bonus ? hent : nullptr;
       z.V = V; z.n = nc; z.n_pad = n_pad; z.cap = d->softcap;
       {
         Timed t(MJ_GRPO_K_DZ, st);
@@ -253,7 +267,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
   if (mode != kBackwardOnly) {
     {
       Timed t(MJ_GRPO_K_REDUCE_LOSS, st);
-      mj::k_reduce_loss<<<1, 1024, 0, st>>>(term, N, loss);
+      mj::k_reduce_loss<<<1, 1024, 0, st>>>(term, eterm, N, d->entropy_coef, loss);
     }
     if ((rc = check_launch("k_reduce_loss"))) return rc;
   }

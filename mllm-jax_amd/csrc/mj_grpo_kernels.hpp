@@ -168,6 +168,9 @@ struct FinalizeArgs {
   float *logp, *lse, *ent;     // chunk origin outputs (ent may be null)
   float* term;                 // per-token loss term
   float* g;                    // [n_pad] dloss/dlogp * gscale, or null (forward only)
+  float ent_coef, inv_ent_cnt; // entropy bonus (0 = off) and its normaliser
+  float* eterm;                // per-token share of the masked mean entropy
+  float *ge, *hent;            // [n_pad] coef*mask*inv_ent_cnt*gscale and H_t, or null (no bonus / forward only)
 };
 
 // block = (64 tokens) x (4 slices of the partial list)
@@ -192,6 +195,7 @@ __global__ __launch_bounds__(256) void k_finalize(FinalizeArgs p) {
   if (ty != 0) return;
   if (t >= p.n) {
     if (p.g != nullptr && t < p.n_pad) p.g[t] = 0.f;
+    if (p.ge != nullptr && t < p.n_pad) p.ge[t] = 0.f;
     return;
   }
   float M = fmaxf(fmaxf(sm[0][tx], sm[1][tx]), fmaxf(sm[2][tx], sm[3][tx]));
@@ -206,8 +210,14 @@ __global__ __launch_bounds__(256) void k_finalize(FinalizeArgs p) {
   const float logp = p.zy[t] - lse;
   p.lse[t] = lse;
   p.logp[t] = logp;
-  if (p.ent != nullptr) p.ent[t] = lse - S / L;   // = -sum p log p  (reference adds 1e-9 inside the log)
+  const float H = lse - S / L;                    // = -sum p log p  (reference adds 1e-9 inside the log)
+  if (p.ent != nullptr) p.ent[t] = H;
   const float mk = p.mask[t];
+  p.eterm[t] = H * mk * p.inv_ent_cnt;
+  if (p.ge != nullptr) {
+    p.ge[t] = p.ent_coef * mk * p.inv_ent_cnt * p.gscale;
+    p.hent[t] = H;
+  }
   float term, g;
   if (p.sft) {
     term = -logp * mk * p.inv_tv;
@@ -248,18 +258,30 @@ __global__ __launch_bounds__(256) void k_coeff_from_saved(const float* logp, con
   g[t] = out * gscale;
 }
 
-// Deterministic single-workgroup sum of the per-token loss terms.
-__global__ __launch_bounds__(1024) void k_reduce_loss(const float* term, int n, float* loss) {
-  __shared__ float sh[1024];
-  float a = 0.f;
-  for (int i = threadIdx.x; i < n; i += 1024) a += term[i];
+// Deterministic single-workgroup sums: loss[1] = masked mean entropy, loss[0] = sum of the
+// per-token policy terms - ent_coef * loss[1].
+__global__ __launch_bounds__(1024) void k_reduce_loss(const float* term, const float* eterm, int n,
+                                                      float ent_coef, float* loss) {
+  __shared__ float sh[1024], se[1024];
+  float a = 0.f, e = 0.f;
+  for (int i = threadIdx.x; i < n; i += 1024) {
+    a += term[i];
+    e += eterm[i];
+  }
   sh[threadIdx.x] = a;
+  se[threadIdx.x] = e;
   __syncthreads();
   for (int o = 512; o > 0; o >>= 1) {
-    if ((int)threadIdx.x < o) sh[threadIdx.x] += sh[threadIdx.x + o];
+    if ((int)threadIdx.x < o) {
+      sh[threadIdx.x] += sh[threadIdx.x + o];
+      se[threadIdx.x] += se[threadIdx.x + o];
+    }
     __syncthreads();
   }
-  if (threadIdx.x == 0) loss[0] = sh[0];
+  if (threadIdx.x == 0) {
+    loss[0] = sh[0] - ent_coef * se[0];
+    loss[1] = se[0];
+  }
 }
 
 // ----------------------------------------------------------------------------- dZ
@@ -267,6 +289,7 @@ struct DzArgs {
   uint16_t* zt;        // [V, ld_z] in: capped logits^T (half); out: dZ^T (bf16)
   int64_t ld_z;
   const float *lse, *g;    // chunk-local (lse valid for t < n, g for t < n_pad)
+  const float *ge, *hent;  // chunk-local entropy-bonus coefficient and H_t, or null
   const int32_t* targets;  // chunk origin
   int V, n, n_pad;
   float cap;
@@ -281,7 +304,8 @@ __global__ __launch_bounds__(256) void k_dz(DzArgs p) {
   const int v0 = blockIdx.y * 64;
   if (t0 >= p.n_pad) return;
   const float inv_cap2 = p.cap > 0.f ? 1.f / (p.cap * p.cap) : 0.f;
-  float lse[8], g[8];
+  const bool bonus = p.ge != nullptr;
+  float lse[8], g[8], ge[8], hent[8];
   int y[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -290,6 +314,8 @@ __global__ __launch_bounds__(256) void k_dz(DzArgs p) {
     lse[i] = in ? p.lse[t] * kLog2e : 0.f;
     g[i] = in ? p.g[t] : 0.f;
     y[i] = in ? p.targets[t] : -1;
+    ge[i] = (bonus && in) ? p.ge[t] : 0.f;
+    hent[i] = (bonus && in) ? p.hent[t] : 0.f;
   }
 #pragma unroll
   for (int step = 0; step < 8; ++step) {
@@ -302,11 +328,13 @@ __global__ __launch_bounds__(256) void k_dz(DzArgs p) {
     for (int i = 0; i < 8; ++i) {
       const uint32_t w = in[i >> 1];
       const float z = f16_bits_to_f32((uint16_t)((i & 1) ? (w >> 16) : (w & 0xffffu)));
-      float d = -__builtin_amdgcn_exp2f(fmaf(z, kLog2e, -lse[i]));
-      if (v == y[i]) d += 1.f;
+      const float t2 = fmaf(z, kLog2e, -lse[i]);          // log2 p
+      const float pr = __builtin_amdgcn_exp2f(t2);
+      float d = (v == y[i]) ? 1.f - pr : -pr;
       d *= g[i];
+      if (bonus) d = fmaf(ge[i] * pr, fmaf(t2, 0.6931471805599453f, hent[i]), d);   // coef * p * (log p + H)
       if (p.cap > 0.f) d *= 1.f - z * z * inv_cap2;
-      if (!(g[i] != 0.f)) d = 0.f;   // masked or padding token: exactly zero, whatever z holds
+      if (!(g[i] != 0.f) && !(ge[i] != 0.f)) d = 0.f;   // masked or padding token: exactly zero, whatever z holds
       const uint32_t b = f32_to_bf16(d);
       if (i & 1) out[i >> 1] |= b << 16; else out[i >> 1] = b;
     }

@@ -5,6 +5,7 @@ Mirrors, for the lm_head + loss part only:
   MLLM_JAX/train_modules/__init__.py:84-192   TrainGRPOModule (inputs / outputs, hyper-parameters)
   plugins/training/update/train_step.py:15-24 loss_fn + jax.value_and_grad(has_aux=True)
   plugins/sft/jax/sft_module.py:22-45         TrainSftModule (masked cross-entropy)
+  plugins/training/ppo/module.py:59-150       PPOActorCriticModule (policy + value + entropy bonus)
 
 torch is used for device memory, streams and autograd plumbing only; all arithmetic on
 [tokens, vocab]-sized data happens in the HIP kernels.  No CPU fallback exists.
@@ -53,7 +54,8 @@ class _Prepared:
 
     def __init__(self, hidden, lm_head, target_ids, old_logps, advantages, mask, *,
                  total_valid_token_count, epsilon_low, epsilon_high, temperature,
-                 final_logit_softcap, seq_shape, chunk_tokens, sft=False, accumulate=False):
+                 final_logit_softcap, seq_shape, chunk_tokens, sft=False, accumulate=False,
+                 entropy_coef=0.0, entropy_token_count=None):
         if hidden.device.type != "cuda":
             raise RuntimeError("grpo_fused_loss needs tensors on an MI355X device (got "
                                f"{hidden.device}); there is no CPU path")
@@ -108,12 +110,16 @@ class _Prepared:
         d.softcap = float(final_logit_softcap or 0.0)
         d.inv_total_valid_tokens = (1.0 / tv) if tv != 0 else float("inf")
         d.grad_loss_scale = 1.0
+        d.entropy_coef = float(entropy_coef)
+        if entropy_coef != 0.0 or entropy_token_count is not None:
+            cnt = float(self.mask.sum().item()) if entropy_token_count is None else float(entropy_token_count)
+            d.inv_entropy_count = 1.0 / (cnt + 1e-8)             # ppo/module.py:77
         d.flags = (_lib.FLAG_SFT if sft else 0) | (_lib.FLAG_DW_ACCUMULATE if accumulate else 0)
         self.desc = d
         self.logp = torch.empty(n, dtype=torch.float32, device=dev)
         self.lse = torch.empty(n, dtype=torch.float32, device=dev)
         self.ent = torch.empty(n, dtype=torch.float32, device=dev)
-        self.loss = torch.empty(1, dtype=torch.float32, device=dev)
+        self.loss = torch.empty(2, dtype=torch.float32, device=dev)   # [loss, masked-mean entropy]
 
     def stream(self) -> int:
         return torch.cuda.current_stream(self.device).cuda_stream
@@ -159,11 +165,14 @@ class _Prepared:
             out["entropy_loss"] = (ent * win).sum(-1) / win.sum(-1)          # :155-157
         if return_token_entropy:
             out["token_entropy"] = self.ent.reshape(shape)
+        if self.desc.inv_entropy_count != 0.0:
+            out["masked_mean_entropy"] = self.loss[1]
         return out
 
 
 _DEFAULTS = dict(total_valid_token_count=None, epsilon_low=0.2, epsilon_high=0.3, temperature=1.0,
-                 final_logit_softcap=None, seq_shape=None, chunk_tokens=None)
+                 final_logit_softcap=None, seq_shape=None, chunk_tokens=None, entropy_coef=0.0,
+                 entropy_token_count=None)
 
 
 def grpo_loss_value_and_grad(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
@@ -174,7 +183,10 @@ def grpo_loss_value_and_grad(hidden, lm_head, target_ids, old_logps, advantages,
     d_hidden is bf16 [N,H]; d_lm_head is float32 [H,V] (the reference's parameter gradients
     are float32).  `accumulate_into` (a float32 [H,V] tensor) makes the kernel add into an
     existing gradient buffer instead of overwriting (grad accumulation, train_step.py:30-33).
-    One fused pass: 6*N*H*V flop, 16-bit logits of at most `chunk_tokens` tokens in the workspace."""
+    One fused pass: 6*N*H*V flop, 16-bit logits of at most `chunk_tokens` tokens in the workspace.
+    `entropy_coef` != 0 subtracts entropy_coef * sum(H_t*mask)/(sum(mask)+1e-8) from the loss
+    (the entropy bonus of plugins/training/ppo/module.py:75-77, :140), gradient included; that
+    entropy is returned as metrics["masked_mean_entropy"]."""
     opts = {**_DEFAULTS, **kw}
     p = _Prepared(hidden, lm_head, target_ids, old_logps, advantages, mask,
                   accumulate=accumulate_into is not None, **opts)
@@ -278,6 +290,94 @@ class TrainGRPOModule:
             epsilon_low=self.epsilon_low, epsilon_high=self.epsilon_high, temperature=self.temperature,
             final_logit_softcap=self.final_logit_softcap, seq_shape=(b, l - 1),
             chunk_tokens=self.chunk_tokens)
+
+
+class PPOActorCriticModule:
+    """Drop-in for the reference's PPOActorCriticModule.__call__ (plugins/training/ppo/module.py:59-150)
+    with the lm_head product, the policy term and the entropy bonus (value and gradient) fused
+    into the HIP kernels.
+
+    `model(input_ids=..., attention_mask=...)` returns the final hidden states [B,L,H];
+    `lm_head` is the [H,V] kernel; `value_head` is (weight [H] or [H,1], bias scalar tensor),
+    the Dense(1, use_bias=True) of module.py:34-39 (each may be a zero-argument callable).
+    The value head is a [B*L,H] x [H] product and a handful of element-wise operations on
+    [B,L] tensors; those run as torch device ops."""
+
+    def __init__(self, model: Callable, lm_head, value_head, temperature: float = 1.0,
+                 epsilon_low: float = 0.2, epsilon_high: float = 0.2, value_coef: float = 0.5,
+                 value_clip_range: Optional[float] = 0.2, entropy_coef: float = 0.0,
+                 final_logit_softcap: Optional[float] = None, chunk_tokens: Optional[int] = None):
+        self.model, self.lm_head, self.value_head = model, lm_head, value_head
+        self.temperature, self.epsilon_low, self.epsilon_high = temperature, epsilon_low, epsilon_high
+        self.value_coef, self.value_clip_range, self.entropy_coef = value_coef, value_clip_range, entropy_coef
+        self.final_logit_softcap, self.chunk_tokens = final_logit_softcap, chunk_tokens
+
+    def _values(self, hidden: torch.Tensor) -> torch.Tensor:
+        wv, bv = self.value_head() if callable(self.value_head) else self.value_head
+        # Dense(1), squeezed (module.py:52); accumulated and kept in float32 (the reference rounds
+        # the result to the activation dtype before casting it back to float32 at :127)
+        return (hidden.float() @ wv.reshape(-1, 1).float()).squeeze(-1) + bv.float()
+
+    def value(self, input_ids, attention_mask) -> torch.Tensor:
+        """module.py:55-57."""
+        return self._values(self.model(input_ids=input_ids, attention_mask=attention_mask))
+
+    @staticmethod
+    def _like(x, ref: torch.Tensor, name: str) -> torch.Tensor:
+        # the [B] / [B,1] / [B,T] broadcasting of module.py:88-94, :108-114, :119-125
+        x = torch.as_tensor(x, device=ref.device)
+        if x.dim() == 1:
+            x = x[:, None]
+        if x.shape != ref.shape:
+            if x.shape[1] == 1:
+                x = x.expand(ref.shape)
+            else:
+                raise ValueError(f"{name} shape {tuple(x.shape)} does not match {tuple(ref.shape)}")
+        return x
+
+    def __call__(self, inputs: Mapping[str, Any]) -> dict:
+        input_ids, labels = inputs["input_ids"], inputs["labels"]
+        hidden = self.model(input_ids=input_ids, attention_mask=inputs["attention_mask"])
+        w = self.lm_head() if callable(self.lm_head) else self.lm_head
+        b, l = input_ids.shape
+        t = l - 1
+        mask = labels[:, 1:].to(torch.float32)                                   # :67
+        value_pred = self._values(hidden)[:, :-1]                                # :104
+        advantages = self._like(inputs["advantages"], value_pred, "advantages")  # :87-94
+        msum = mask.sum()
+        tv = inputs.get("total_valid_token_count")
+        p = _Prepared(hidden[:, :-1, :].reshape(b * t, -1), w, input_ids[:, 1:].reshape(-1),
+                      inputs.get("old_per_token_logps"), advantages.reshape(-1), mask.reshape(-1),
+                      total_valid_token_count=float(tv) if tv is not None else float(msum.item()),
+                      epsilon_low=self.epsilon_low, epsilon_high=self.epsilon_high,
+                      temperature=self.temperature, final_logit_softcap=self.final_logit_softcap,
+                      seq_shape=(b, t), chunk_tokens=self.chunk_tokens, entropy_coef=self.entropy_coef,
+                      entropy_token_count=float(msum.item()) if self.entropy_coef != 0.0 or tv is None else None)
+        want = torch.is_grad_enabled() and (hidden.requires_grad or w.requires_grad)
+        fused = _FusedLossFn.apply(hidden[:, :-1, :].reshape(b * t, -1), w, p, want)   # policy - coef * entropy
+        entropy = (p.ent.reshape(b, t) * mask).sum() / (msum + 1e-8)             # :77
+        policy_loss = (fused + self.entropy_coef * entropy).detach()
+
+        returns = inputs.get("returns")
+        if returns is None:
+            returns = advantages + value_pred                                    # :107 (not detached)
+        returns = self._like(returns, value_pred, "returns")
+        old_values = inputs.get("old_values", inputs.get("values"))
+        if old_values is None:
+            old_values = value_pred.detach()                                     # :118
+        old_values = self._like(old_values, value_pred, "old_values")
+        vp, rt, ov = value_pred.float(), returns.float(), old_values.float()
+        if self.value_clip_range is not None:
+            c = float(self.value_clip_range)
+            clipped = ov + torch.clamp(vp - ov, -c, c)
+            value_loss = torch.maximum((vp - rt) ** 2, (clipped - rt) ** 2)      # :133-134
+        else:
+            value_loss = (vp - rt) ** 2
+        value_loss = (value_loss * mask).sum() / p.tv                            # :138
+        loss = fused + float(self.value_coef) * value_loss                       # :140
+        return {"loss": loss, "policy_loss": policy_loss, "value_loss": value_loss, "entropy": entropy,
+                "value_pred_mean": vp.mean(), "return_mean": rt.mean(),
+                "per_token_logps": p.logp.reshape(b, t)}
 
 
 def loss_and_metrics(module: Callable[[Mapping[str, Any]], dict], inputs: Mapping[str, Any]):

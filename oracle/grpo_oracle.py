@@ -11,7 +11,7 @@ reference's un-fused jnp loss:
   deprecated/MLLM_JAX/language/gemma/transformer.py:337-339 (final-logit softcap)
   plugins/training/update/train_step.py:15-24  (value_and_grad -> closed-form backward)
   plugins/training/advantage/grpo.py:28-52     (group-normalised advantages)
-  plugins/training/ppo/module.py:59-150        (actor-critic twin; policy part)
+  plugins/training/ppo/module.py:59-150        (actor-critic twin: policy + value + entropy bonus)
   plugins/sft/jax/sft_module.py:22-45          (masked cross-entropy)
 
 The arithmetic itself lives in un-vendored JAX (jax.nn.log_softmax, jax.nn.softmax,
@@ -143,6 +143,80 @@ def grpo_loss(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
         out["d_hidden"] = dz @ w.T
         out["d_lm_head"] = h.T @ dz
         out["dlogp"] = g
+    return out
+
+
+def ppo_actor_critic_loss(hidden, lm_head, value_w, value_b, target_ids, old_logps, advantages, mask, *,
+                          returns=None, old_values=None, total_valid_token_count=None,
+                          epsilon_low=0.2, epsilon_high=0.2, value_coef=0.5, value_clip_range=0.2,
+                          entropy_coef=0.0, final_logit_softcap=None, with_grads=True):
+    """PPOActorCriticModule.__call__ (plugins/training/ppo/module.py:59-150) on flattened,
+    already shifted tokens, float64, with closed-form gradients.
+
+      entropy     = sum(H_t * mask) / (sum(mask) + 1e-8)                       (:75-77)
+      policy_loss = sum(-min(ratio*adv, clip(ratio)*adv) * mask) / tvtc        (:84-102)
+      returns     = advantages + value_pred when absent (NOT detached, :107)
+      old_values  = stop_gradient(value_pred) when absent                      (:118)
+      value_loss  = sum(max((v-R)^2, (old + clip(v-old, +-c) - R)^2) * mask) / tvtc   (:131-138)
+      loss        = policy_loss + value_coef*value_loss - entropy_coef*entropy (:140)
+
+    value_pred = hidden @ value_w + value_b is the Dense(1) of :34-39, :52.  Where the two
+    arguments of max() are equal each receives half the cotangent (lax.max's JVP)."""
+    h = np.asarray(hidden, np.float64)
+    w = np.asarray(lm_head, np.float64)
+    wv = np.asarray(value_w, np.float64).reshape(-1)
+    bv = float(np.asarray(value_b, np.float64).reshape(()))
+    n = h.shape[0]
+    y = np.asarray(target_ids).astype(np.int64)
+    m = np.asarray(mask, np.float64)
+    adv = np.asarray(advantages, np.float64)
+    cap = float(final_logit_softcap) if final_logit_softcap else None
+    z_raw = h @ w
+    z = cap * np.tanh(z_raw / cap) if cap else z_raw
+    logp, lse, ent = token_logps_and_entropy(z, y, 1.0)
+    cnt = m.sum() + 1e-8
+    entropy = (ent * m).sum() / cnt
+    tv = float(m.sum()) if total_valid_token_count is None else float(total_valid_token_count)
+    policy_loss, g = policy_loss_terms(logp, old_logps, adv, m, tv, epsilon_low, epsilon_high)
+
+    vp = h @ wv + bv
+    rt_free = returns is None
+    rt = adv + vp if rt_free else np.asarray(returns, np.float64)
+    ov = vp.copy() if old_values is None else np.asarray(old_values, np.float64)
+    a = (vp - rt) ** 2
+    da = 2.0 * (vp - rt) * (0.0 if rt_free else 1.0)
+    if value_clip_range is not None:
+        c = float(value_clip_range)
+        delta = vp - ov
+        clipped = ov + np.clip(delta, -c, c)
+        inside = (np.abs(delta) <= c).astype(np.float64)
+        b = (clipped - rt) ** 2
+        db = 2.0 * (clipped - rt) * (inside - (1.0 if rt_free else 0.0))
+        vl = np.maximum(a, b)
+        dvl = np.where(a > b, da, np.where(a < b, db, 0.5 * (da + db)))
+    else:
+        vl, dvl = a, da
+    value_loss = (vl * m).sum() / tv
+    loss = policy_loss + float(value_coef) * value_loss - float(entropy_coef) * entropy
+    out = {"loss": loss, "policy_loss": policy_loss, "value_loss": value_loss, "entropy": entropy,
+           "value_pred_mean": vp.mean(), "return_mean": rt.mean(), "per_token_logps": logp,
+           "token_entropy": ent, "value_pred": vp}
+    if with_grads:
+        p = np.exp(z - lse[:, None])
+        dz = -p
+        dz[np.arange(n), y] += 1.0
+        dz *= g[:, None]
+        # d(-coef*entropy)/dz_j = coef*mask/cnt * p_j * (a_j - sum_i p_i a_i) with
+        # a_i = dH/dp_i negated = log(p_i + 1e-9) + p_i/(p_i + 1e-9)
+        ai = np.log(p + 1e-9) + p / (p + 1e-9)
+        dz += (float(entropy_coef) * m / cnt)[:, None] * p * (ai - (p * ai).sum(-1, keepdims=True))
+        if cap:
+            dz *= 1.0 - (z / cap) ** 2
+        dv = float(value_coef) * dvl * m / tv
+        out["d_hidden"] = dz @ w.T + dv[:, None] * wv[None, :]
+        out["d_lm_head"] = h.T @ dz
+        out["d_value_w"] = h.T @ dv
+        out["d_value_b"] = dv.sum()
     return out
 
 

@@ -39,8 +39,8 @@ def test_header_symbols_are_exported(lib):
 
 
 def test_desc_layout_matches_header(lib):
-    # 6 x int64 + 6 x float + 2 x uint32
-    assert C.sizeof(lib.MjGrpoDesc) == 6 * 8 + 6 * 4 + 2 * 4
+    # 6 x int64 + 6 x float + 2 x uint32 + 2 x float
+    assert C.sizeof(lib.MjGrpoDesc) == 6 * 8 + 6 * 4 + 2 * 4 + 2 * 4
 
 
 def test_workspace_sizes_scale_with_chunk(lib):
@@ -58,6 +58,7 @@ def test_workspace_sizes_scale_with_chunk(lib):
     (dict(vocab=508, ld_w=508), 3), (dict(hidden=60, ld_hidden=60), 3), (dict(ld_hidden=68), 3),
     (dict(temperature=0.7), 5), (dict(softcap=-1.0), 5), (dict(chunk_tokens=-5), 2),
     (dict(inv_total_valid_tokens=float("inf")), 2),
+    (dict(entropy_coef=float("nan")), 2), (dict(inv_entropy_count=-1.0), 2),
 ])
 def test_bad_descriptors(lib, kw, code):
     with pytest.raises(lib.MjGrpoError) as e:

@@ -228,3 +228,111 @@ def test_chunked_torch_oracle_matches_float64(rng):
     np.testing.assert_allclose(b["token_entropy"], a["token_entropy"], atol=1e-5)
     np.testing.assert_allclose(b["d_hidden"], a["d_hidden"], atol=1e-6)
     np.testing.assert_allclose(b["d_lm_head"], a["d_lm_head"], atol=1e-6)
+
+
+# --------------------------------------------------------------------------- PPO actor-critic
+def _ppo_autograd(hid, w, wv, bv, y, old, adv, mask, returns, old_values, tv, el, eh, vc, clip, ec, cap):
+    """Library-routine restatement (torch float64 autograd) of the actor-critic loss; written
+    against plugins/training/ppo/module.py:66-140, not against the oracle."""
+    t = lambda x: torch.tensor(np.asarray(x, np.float64))
+    hid_t, w_t, wv_t = t(hid).requires_grad_(), t(w).requires_grad_(), t(wv).requires_grad_()
+    bv_t = t(bv).requires_grad_()
+    z = hid_t @ w_t
+    if cap:
+        z = cap * torch.tanh(z / cap)
+    lsm = torch.log_softmax(z, -1)
+    logp = lsm.gather(-1, torch.tensor(y)[:, None])[:, 0]
+    probs = torch.softmax(z, -1)
+    ent_t = -(probs * torch.log(probs + 1e-9)).sum(-1)
+    m = t(mask)
+    entropy = (ent_t * m).sum() / (m.sum() + 1e-8)
+    oldt = logp.detach() if old is None else t(old)
+    ratio = torch.exp(logp - oldt)
+    a = t(adv)
+    ppo = torch.minimum(ratio * a, torch.clamp(ratio, 1 - el, 1 + eh) * a)
+    tvt = m.sum() if tv is None else tv
+    policy = (-ppo * m).sum() / tvt
+    vp = hid_t @ wv_t + bv_t
+    rt = a + vp if returns is None else t(returns)
+    ov = vp.detach() if old_values is None else t(old_values)
+    if clip is not None:
+        vclipped = ov + torch.clamp(vp - ov, -clip, clip)
+        vl = torch.maximum((vp - rt) ** 2, (vclipped - rt) ** 2)
+    else:
+        vl = (vp - rt) ** 2
+    vloss = (vl * m).sum() / tvt
+    loss = policy + vc * vloss - ec * entropy
+    loss.backward()
+    return dict(loss=loss.item(), policy_loss=policy.item(), value_loss=vloss.item(), entropy=entropy.item(),
+                d_hidden=hid_t.grad.numpy(), d_lm_head=w_t.grad.numpy(), d_value_w=wv_t.grad.numpy(),
+                d_value_b=bv_t.grad.item())
+
+
+@pytest.mark.parametrize("case", ["defaults", "given_returns_values", "no_clip", "entropy_softcap", "off_policy_tvtc"])
+def test_ppo_actor_critic_matches_float64_autograd(rng, case):
+    hid, w, y, adv_seq, mask = _inputs(rng)
+    n, h = hid.shape
+    wv, bv = rng.standard_normal(h) * 0.3, 0.17
+    adv = rng.standard_normal(n)                     # per-token advantages (GAE), module.py:87-94
+    kw = dict(returns=None, old_values=None, tv=None, el=0.2, eh=0.2, vc=0.5, clip=0.2, ec=0.0, cap=None)
+    old = None
+    if case == "given_returns_values":
+        vp = hid @ wv + bv
+        kw.update(returns=vp + rng.standard_normal(n), old_values=vp + 0.3 * rng.standard_normal(n), ec=0.01)
+    elif case == "no_clip":
+        kw.update(returns=rng.standard_normal(n), clip=None, vc=1.3)
+    elif case == "entropy_softcap":
+        kw.update(ec=0.05, cap=3.0, returns=rng.standard_normal(n))
+    elif case == "off_policy_tvtc":
+        z = hid @ w
+        old = sps.log_softmax(z, -1)[np.arange(n), y] + 0.25 * rng.standard_normal(n)
+        kw.update(tv=23.0, ec=0.02, el=0.1, eh=0.3, old_values=rng.standard_normal(n))
+    ref = _ppo_autograd(hid, w, wv, bv, y, old, adv, mask, **kw)
+    got = O.ppo_actor_critic_loss(hid, w, wv, bv, y, old, adv, mask, returns=kw["returns"],
+                                  old_values=kw["old_values"], total_valid_token_count=kw["tv"],
+                                  epsilon_low=kw["el"], epsilon_high=kw["eh"], value_coef=kw["vc"],
+                                  value_clip_range=kw["clip"], entropy_coef=kw["ec"],
+                                  final_logit_softcap=kw["cap"])
+    for k in ("loss", "policy_loss", "value_loss", "entropy", "d_value_b"):
+        np.testing.assert_allclose(got[k], ref[k], rtol=1e-10, atol=1e-12, err_msg=k)
+    for k in ("d_hidden", "d_lm_head", "d_value_w"):
+        np.testing.assert_allclose(got[k], ref[k], rtol=1e-9, atol=1e-12, err_msg=k)
+
+
+def test_ppo_default_value_loss_is_mean_squared_advantage(rng):
+    # returns = adv + v and old_values = sg(v): both branches equal adv^2, whatever the value head is,
+    # and the value head receives no gradient (module.py:107, :118, :133-134)
+    hid, w, y, _, mask = _inputs(rng)
+    n, h = hid.shape
+    adv = rng.standard_normal(n)
+    out = O.ppo_actor_critic_loss(hid, w, rng.standard_normal(h), 0.4, y, None, adv, mask, value_coef=0.7)
+    np.testing.assert_allclose(out["value_loss"], (adv ** 2 * mask).sum() / mask.sum(), rtol=1e-12)
+    np.testing.assert_allclose(out["d_value_w"], 0.0, atol=1e-12)
+    np.testing.assert_allclose(out["policy_loss"], -(adv * mask).sum() / mask.sum(), rtol=1e-12)   # ratio == 1
+
+
+def test_ppo_entropy_gradient_finite_differences(rng):
+    # only the entropy bonus active: advantages zero, value_coef zero
+    hid, w, y, _, mask = _inputs(rng, n=6, h=5, v=11, b=3)
+    n, h = hid.shape
+    wv = np.zeros(h)
+    f = lambda hh, ww: O.ppo_actor_critic_loss(hh, ww, wv, 0.0, y, None, np.zeros(n), mask, value_coef=0.0,
+                                               entropy_coef=1.0, with_grads=False)["loss"]
+    out = O.ppo_actor_critic_loss(hid, w, wv, 0.0, y, None, np.zeros(n), mask, value_coef=0.0, entropy_coef=1.0)
+    np.testing.assert_allclose(out["loss"], -out["entropy"], rtol=1e-12)
+    e = 1e-6
+    for (i, j) in [(0, 0), (2, 3), (5, 4)]:
+        d = np.zeros_like(hid); d[i, j] = e
+        np.testing.assert_allclose(out["d_hidden"][i, j], (f(hid + d, w) - f(hid - d, w)) / (2 * e), rtol=1e-5, atol=1e-9)
+    for (i, j) in [(0, 0), (3, 7), (4, 10)]:
+        d = np.zeros_like(w); d[i, j] = e
+        np.testing.assert_allclose(out["d_lm_head"][i, j], (f(hid, w + d) - f(hid, w - d)) / (2 * e), rtol=1e-5, atol=1e-9)
+
+
+def test_ppo_uniform_policy_has_maximal_entropy_and_no_entropy_gradient():
+    v, n, h = 64, 4, 3
+    hid = np.ones((n, h)); w = np.zeros((h, v))
+    out = O.ppo_actor_critic_loss(hid, w, np.zeros(h), 0.0, np.arange(n), None, np.zeros(n), np.ones(n),
+                                  entropy_coef=0.5, value_coef=0.0)
+    np.testing.assert_allclose(out["entropy"], np.log(v), atol=1e-6)       # 1e-9 inside the log, module.py:76
+    np.testing.assert_allclose(out["d_lm_head"], 0.0, atol=1e-15)
