@@ -12,7 +12,9 @@ torch is used for device memory, streams and autograd plumbing only; all arithme
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
+import threading
 from typing import Any, Callable, Mapping, Optional
 
 import torch
@@ -191,19 +193,57 @@ def grpo_loss_value_and_grad(hidden, lm_head, target_ids, old_logps, advantages,
     p = _Prepared(hidden, lm_head, target_ids, old_logps, advantages, mask,
                   accumulate=accumulate_into is not None, **opts)
     if accumulate_into is not None:
-        if accumulate_into.dtype != torch.float32 or tuple(accumulate_into.shape) != (p.h, p.v) \
-                or accumulate_into.stride(1) != 1 or accumulate_into.stride(0) != p.w.stride(0):
-            raise ValueError("accumulate_into must be a float32 [H,V] tensor laid out like lm_head")
+        _check_accumulator(accumulate_into, p)
     d_h, d_w = p.forward_backward(accumulate_into)
     return p.metrics(return_token_entropy), (d_h.reshape(hidden.shape), d_w)
+
+
+def _check_accumulator(buf: torch.Tensor, p: "_Prepared") -> None:
+    if buf.dtype != torch.float32 or tuple(buf.shape) != (p.h, p.v) \
+            or buf.stride(1) != 1 or buf.stride(0) != p.w.stride(0) or buf.device != p.device:
+        raise ValueError("the lm_head gradient accumulator must be a float32 [H,V] device tensor laid out like lm_head")
+
+
+class _AccumulateTarget(threading.local):
+    buffer: Optional[torch.Tensor] = None
+    uses: int = 0
+
+
+_accumulate_target = _AccumulateTarget()
+
+
+@contextlib.contextmanager
+def accumulate_lm_head_grad_into(buffer: torch.Tensor):
+    """Within this context every differentiable fused-loss call ADDS its lm_head gradient into
+    `buffer` (float32 [H,V]) inside the dW kernel and hands autograd no lm_head gradient: the
+    grad-accumulation `ga + g` of plugins/training/update/train_step.py:30-33 without a
+    separate [H,V] gradient tensor or a pass over it.  The loss must be terminal (it is
+    differentiated with upstream gradient 1, as training_step does); yields a counter object
+    whose `.uses` says how many calls accumulated."""
+    prev, prev_uses = _accumulate_target.buffer, _accumulate_target.uses
+    _accumulate_target.buffer, _accumulate_target.uses = buffer, 0
+    try:
+        yield _accumulate_target
+    finally:
+        _accumulate_target.buffer, _accumulate_target.uses = prev, prev_uses
 
 
 class _FusedLossFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, lm_head, prepared: _Prepared, want_grad: bool):
+        ctx.direct = False
         if want_grad:
-            d_h, d_w = prepared.forward_backward()
-            ctx.save_for_backward(d_h, d_w)
+            buf = _accumulate_target.buffer if lm_head.requires_grad else None
+            if buf is not None:
+                _check_accumulator(buf, prepared)
+                prepared.desc.flags |= _lib.FLAG_DW_ACCUMULATE
+                d_h, _ = prepared.forward_backward(buf)
+                _accumulate_target.uses += 1
+                ctx.direct = True
+                ctx.save_for_backward(d_h)
+            else:
+                d_h, d_w = prepared.forward_backward()
+                ctx.save_for_backward(d_h, d_w)
             ctx.shapes = (hidden.shape, hidden.dtype, lm_head.dtype)
         else:
             prepared.forward()
@@ -211,10 +251,14 @@ class _FusedLossFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_loss):
-        d_h, d_w = ctx.saved_tensors
         shape, h_dtype, w_dtype = ctx.shapes
+        if ctx.direct:
+            (d_h,) = ctx.saved_tensors
+            gw = None                      # already added into the accumulator by the dW kernel
+        else:
+            d_h, d_w = ctx.saved_tensors
+            gw = (d_w * grad_loss).to(w_dtype)
         gh = (d_h * grad_loss.to(d_h.dtype)).reshape(shape).to(h_dtype)
-        gw = (d_w * grad_loss).to(w_dtype)
         return gh, gw, None, None
 
 

@@ -102,7 +102,7 @@ def _run_case(seed, b, l, h, v, *, old_noise=0.0, returns=False, old_values=Fals
 def test_defaults_value_loss_is_masked_mean_squared_advantage():
     out, ref = _run_case(3, 3, 41, 64, 1000)
     # returns = adv + v, old_values = sg(v): the value head receives no gradient (module.py:107, :118)
-    assert abs(float(out["value_loss"]) - ref["value_loss"]) <= 1e-5 * ref["value_loss"]
+    assert abs(float(out["value_loss"].detach()) - ref["value_loss"]) <= 1e-5 * ref["value_loss"]
 
 
 @pytest.mark.parametrize("coef", [0.01, 0.5])
