@@ -121,7 +121,7 @@ def main() -> int:
         "data": "synthetic",
         "config": {"workload": f"BASELINE configs[{args.config}] {cfg.name}: fused GRPO loss fwd+bwd, "
                                f"{n} tokens x hidden {h} x vocab {v}", "tokens": n, "hidden": h, "vocab": v,
-                   "chunk_tokens": args.chunk_tokens or 8192, "softcap": cfg.softcap,
+                   "chunk_tokens": args.chunk_tokens or min(16384, n), "softcap": cfg.softcap,
                    "eps": [cfg.eps_low, cfg.eps_high]},
         "pct_bf16_mfma_peak": round(100.0 * mfu, 2),
         "algorithmic_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 1),

@@ -64,24 +64,27 @@ MJ_DEV __amdgpu_buffer_rsrc_t make_rsrc_wave(const void* p, int64_t bytes) {
 // s_waitcnt with only the LDS/scalar counter constrained (gfx9 encoding).
 MJ_DEV void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc07f); }
 
-// Maps a linear workgroup id to a tile so that (a) the 32 workgroups that land on one
-// XCD at a time (ids congruent mod 8 go to the same XCD) form a GM x GN block of tiles
-// sharing operand slices in that XCD's L2, and (b) consecutive blocks -- the ones the eight
-// XCDs work on at the same time -- walk along N first (n_first) or along M first.
-template <int GM, int GN>
+// Maps a linear work-item id to a tile (and a k-split) so that (a) the 32 items that the
+// workgroups of one XCD work on at the same time (ids congruent mod 8 go to the same XCD) form a
+// 2^lgm x 2^(5-lgm) block of tiles sharing operand slices in that XCD's L2, and (b) consecutive
+// blocks -- the ones the eight XCDs work on at the same time -- walk along N first (n_first) or
+// along M first.  The blocks of all k-splits form one list.
 struct TileMap {
-  int tiles_m, tiles_n, sb_m, sb_n, n_first;
-  __host__ __device__ TileMap(int tm, int tn, int n_first_ = 0)
-      : tiles_m(tm), tiles_n(tn), sb_m((tm + GM - 1) / GM), sb_n((tn + GN - 1) / GN), n_first(n_first_) {}
-  __host__ __device__ int items() const { return ((sb_m * sb_n + 7) / 8) * 8 * (GM * GN); }
-  __host__ int grid() const { return items(); }
-  MJ_DEV bool tile(int pid, int& tm, int& tn) const {
+  int tiles_m, tiles_n, sb_m, sb_n, n_first, lgm, splits;
+  __host__ __device__ TileMap(int tm, int tn, int n_first_ = 0, int lgm_ = 2, int splits_ = 1)
+      : tiles_m(tm), tiles_n(tn), sb_m((tm + (1 << lgm_) - 1) >> lgm_),
+        sb_n((tn + (1 << (5 - lgm_)) - 1) >> (5 - lgm_)), n_first(n_first_), lgm(lgm_), splits(splits_) {}
+  __host__ __device__ int blocks() const { return sb_m * sb_n * splits; }
+  __host__ __device__ int items() const { return (blocks() + 7) / 8 * 8 * 32; }
+  MJ_DEV bool tile(int pid, int& tm, int& tn, int& split) const {
     const int xcd = pid & 7, q = pid >> 3;
-    const int sb = (q / (GM * GN)) * 8 + xcd, within = q % (GM * GN);
-    if (sb >= sb_m * sb_n) return false;
+    const int sbg = (q >> 5) * 8 + xcd, within = q & 31, per = sb_m * sb_n;
+    if (sbg >= per * splits) return false;
+    split = sbg / per;
+    const int sb = sbg - split * per;
     const int bm = n_first ? sb / sb_n : sb % sb_m, bn = n_first ? sb % sb_n : sb / sb_m;
-    tm = bm * GM + within % GM;
-    tn = bn * GN + within / GM;
+    tm = (bm << lgm) + (within & ((1 << lgm) - 1));
+    tn = (bn << (5 - lgm)) + (within >> lgm);
     return tm < tiles_m && tn < tiles_n;
   }
 };

@@ -46,7 +46,7 @@ struct Timed {
 };
 
 constexpr int BM = 256, BN = 256;          // tile of all three contractions
-constexpr int64_t kDefaultChunk = 8192;    // tokens whose logits live in the workspace at once
+constexpr int64_t kDefaultChunk = 16384;   // tokens whose logits live in the workspace at once
 
 inline int64_t rup(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 
@@ -196,9 +196,9 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       a.zt = bwd ? zt : nullptr; a.ld_z = p.n_pad;
       a.pm = pm; a.pl = pl; a.ps = ps; a.ld_p = p.n_pad;
       a.targets = targets + c0; a.zy = zy + c0;
-      mj::TileMap<4, 8> map((V + BM - 1) / BM, (nc + BN - 1) / BN, 1);
+      const mj::TileMap map((V + BM - 1) / BM, (nc + BN - 1) / BN, 1);
       Timed t(MJ_GRPO_K_LOGITS_STATS, st);
-      mj::k_logits_stats<BM, BN><<<map.grid(), mj::kThreads, lds, st>>>(a, map);
+      mj::k_logits_stats<BM, BN><<<map.items(), mj::kThreads, lds, st>>>(a, map);
     }
     if (mode != kBackwardOnly) {
       mj::FinalizeArgs f;
@@ -239,10 +239,10 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       h.splits = p.dh_splits; h.k_per_split = (int)p.dh_k_per_split;
       h.dh = (uint16_t*)d_hidden + c0 * d->ld_hidden; h.ld_dh = d->ld_hidden;
       h.part = part;
-      mj::TileMap<4, 8> mh((nc + BM - 1) / BM, (H + BN - 1) / BN, 0);
+      const mj::TileMap mh((nc + BM - 1) / BM, (H + BN - 1) / BN, 0, 2, h.splits);
       {
         Timed t(MJ_GRPO_K_DHIDDEN, st);
-        mj::k_dhidden<BM, BN><<<mh.grid() * h.splits, mj::kThreads, lds, st>>>(h, mh);
+        mj::k_dhidden<BM, BN><<<mh.items(), mj::kThreads, lds, st>>>(h, mh);
       }
       if (h.splits > 1) {
         const int64_t work = (int64_t)nc * (H / 4);
@@ -256,10 +256,10 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       w.H = H; w.V = V; w.n = nc;
       w.dw = d_w; w.ld_dw = d->ld_w;
       w.accumulate = (c0 > 0 || (d->flags & MJ_GRPO_FLAG_DW_ACCUMULATE)) ? 1 : 0;
-      mj::TileMap<4, 8> mw((V + BM - 1) / BM, (H + BN - 1) / BN, 0);
+      const mj::TileMap mw((V + BM - 1) / BM, (H + BN - 1) / BN, 0);
       {
         Timed t(MJ_GRPO_K_DW, st);
-        mj::k_dw<BM, BN><<<mw.grid(), mj::kThreads, lds, st>>>(w, mw);
+        mj::k_dw<BM, BN><<<mw.items(), mj::kThreads, lds, st>>>(w, mw);
       }
     }
     if ((rc = check_launch("chunk kernels"))) return rc;
@@ -354,6 +354,6 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
 }  // extern "C"
 
 // Explicit instantiations of the tile kernels used above.
-template __global__ void mj::k_logits_stats<256, 256>(mj::LogitsArgs, mj::TileMap<4, 8>);
-template __global__ void mj::k_dhidden<256, 256>(mj::DhArgs, mj::TileMap<4, 8>);
-template __global__ void mj::k_dw<256, 256>(mj::DwArgs, mj::TileMap<4, 8>);
+template __global__ void mj::k_logits_stats<256, 256>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_dhidden<256, 256>(mj::DhArgs, mj::TileMap);
+template __global__ void mj::k_dw<256, 256>(mj::DwArgs, mj::TileMap);

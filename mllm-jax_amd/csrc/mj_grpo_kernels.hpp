@@ -54,6 +54,9 @@ MJ_DEV void store_b32(float v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t
 MJ_DEV void store_b128(f32x4 v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
   __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff, soff, 0);
 }
+MJ_DEV float load_b32(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
 MJ_DEV f32x4 load_b128(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
   return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
@@ -74,11 +77,11 @@ struct LogitsArgs {
 };
 
 template <int BM, int BN>
-__global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap<4, 8> map) {
+__global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap map) {
   using G = GemmTN<BM, BN, kKRow, kRowK>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  int tm, tn;
-  if (!map.tile(blockIdx.x, tm, tn)) return;
+  int tm, tn, split;
+  if (!map.tile(blockIdx.x, tm, tn, split)) return;
   const int m0 = tm * BM, n0 = tn * BN;
   G g;
   g.run(p.w + m0, p.V - m0, p.ld_w, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0, p.ld_hid, p.H, smem);
@@ -97,17 +100,29 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
     const int col = n0 + wn * G::WN + ni * 32 + l31;
+    // Softcap and the stand-in for rows past V are rare, wave-uniform cases: each sits behind a
+    // real scalar branch (the empty asm keeps the compiler from flattening it into per-element
+    // selects, which would cost an exp and a reciprocal per logit whether or not a cap is set).
+    if (p.cap > 0.f) {
+      asm volatile("");
+#pragma unroll
+      for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) g.acc[mi][ni][r] = softcap_apply(g.acc[mi][ni][r], p.cap, inv_cap);
+    }
+    if (tail) {
+      asm volatile("");
+#pragma unroll
+      for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if ((vbase + mi * 32 + (r >> 2) * 8 + (r & 3)) >= p.V) g.acc[mi][ni][r] = kNegBig;
+    }
     float mx = kNegBig;
 #pragma unroll
     for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float z = g.acc[mi][ni][r];
-        if (p.cap > 0.f) z = softcap_apply(z, p.cap, inv_cap);
-        if (tail && (vbase + mi * 32 + (r >> 2) * 8 + (r & 3)) >= p.V) z = kNegBig;
-        g.acc[mi][ni][r] = z;
-        mx = fmaxf(mx, z);
-      }
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, g.acc[mi][ni][r]);
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     float l = 0.f, s = 0.f;
     const float mxl = mx * kLog2e;
@@ -355,13 +370,11 @@ struct DhArgs {
 };
 
 template <int BM, int BN>
-__global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap<4, 8> map) {
+__global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
   using G = GemmTN<BM, BN, kKRow, kRowK>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  const int per = map.items();
-  const int split = blockIdx.x / per;
-  int tm, tn;
-  if (!map.tile(blockIdx.x - split * per, tm, tn)) return;
+  int tm, tn, split;
+  if (!map.tile(blockIdx.x, tm, tn, split)) return;
   const int m0 = tm * BM, n0 = tn * BN;
   const int k0 = split * p.k_per_split;
   const int klen = min(p.V - k0, p.k_per_split);
@@ -431,11 +444,11 @@ struct DwArgs {
 // Tile of dW^T: rows = vocab (MFMA row direction), columns = hidden (lanes).  A lane's four
 // consecutive accumulator rows are four consecutive floats of one dW row: 16-byte accesses.
 template <int BM, int BN>
-__global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap<4, 8> map) {
+__global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
   using G = GemmTN<BM, BN, kRowK, kKRow>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  int tm, tn;
-  if (!map.tile(blockIdx.x, tm, tn)) return;
+  int tm, tn, split;
+  if (!map.tile(blockIdx.x, tm, tn, split)) return;
   const int m0 = tm * BM, n0 = tn * BN;
   G g;
   g.run(p.dzt + (int64_t)m0 * p.ld_z, p.V - m0, p.ld_z, p.hid + n0, p.H - n0, p.ld_hid, p.n, smem);
@@ -453,16 +466,29 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap<4, 8> map) {
   for (int ni = 0; ni < G::NI; ++ni) {
     const uint32_t lane_off = (uint32_t)((ni * 32 + l31) * ld4 + lhi * 16);
 #pragma unroll
-    for (int mi = 0; mi < G::MI; ++mi)
+    for (int mh = 0; mh < G::MI; mh += 2) {
+      // when accumulating, the eight loads of this half are issued before the first store (a store
+      // between two loads would order the second behind it: one memory round trip per 16 bytes)
+      f32x4 a[2][4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int vv = mi * 32 + q * 8;
-        const uint32_t voff = (vv + lhi * 4) < vleft ? lane_off : kOob;
-        f32x4 a = {g.acc[mi][ni][q * 4], g.acc[mi][ni][q * 4 + 1], g.acc[mi][ni][q * 4 + 2],
-                   g.acc[mi][ni][q * 4 + 3]};
-        if (p.accumulate) a += load_b128(rs, voff, (uint32_t)vv * 4);
-        store_b128(a, rs, voff, (uint32_t)vv * 4);
-      }
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int vv = (mh + mi) * 32 + q * 8;
+          if (p.accumulate) a[mi][q] = load_b128(rs, (vv + lhi * 4) < vleft ? lane_off : kOob, (uint32_t)vv * 4);
+          else a[mi][q] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int vv = (mh + mi) * 32 + q * 8;
+          const uint32_t voff = (vv + lhi * 4) < vleft ? lane_off : kOob;
+          const f32x4 c = {g.acc[mh + mi][ni][q * 4], g.acc[mh + mi][ni][q * 4 + 1], g.acc[mh + mi][ni][q * 4 + 2],
+                           g.acc[mh + mi][ni][q * 4 + 3]};
+          store_b128(c + a[mi][q], rs, voff, (uint32_t)vv * 4);
+        }
+    }
   }
 }
 
