@@ -31,6 +31,33 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
+def _vendor_gemm(torch, hidden, w, n, h, v, reps=5):
+    dev = hidden.device
+    out = {}
+    dz = torch.empty(n, v, dtype=torch.bfloat16, device=dev).normal_(0, 0.01)
+    cases = {"logits": (lambda o: torch.matmul(hidden, w, out=o), (n, v)),
+             "dhidden": (lambda o: torch.matmul(dz, w.t(), out=o), (n, h)),
+             "dw": (lambda o: torch.matmul(hidden.t(), dz, out=o), (h, v))}
+    total = 0.0
+    for name, (fn, shape) in cases.items():
+        o = torch.empty(shape, dtype=torch.bfloat16, device=dev)
+        for _ in range(2):
+            fn(o)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn(o)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        total += ms
+        out[name] = {"ms": round(ms, 3), "tflops": round(2.0 * n * h * v / ms / 1e9, 1)}
+        del o
+    out["sum_ms"] = round(total, 3)
+    out["note"] = "torch.matmul (hipBLASLt) bf16 in, bf16 out, same shapes, same GPU; products only"
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -38,8 +65,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (default 2)")
     ap.add_argument("--chunk-tokens", type=int, default=0)
-    ap.add_argument("--cpu-sample-tokens", type=int, default=4096)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-vendor-gemm", action="store_true",
+                    help="skip timing the three bare bf16 products with the vendor GEMM (torch.matmul = hipBLASLt)")
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known traffic, to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -129,6 +158,14 @@ def main() -> int:
         "roofline": roofline,
         "kernel_ms_per_step": {k: round(v_[0] / args.steps, 3) for k, v_ in prof.items()},
     }
+
+    if not args.no_vendor_gemm:
+        # Context for the roofline fraction: what the vendor's tuned GEMM reaches on this very
+        # GPU for the three bare products (no softmax statistics, no loss, bf16 outputs).
+        del metrics, grads
+        M.release_workspaces()
+        torch.cuda.empty_cache()
+        line["vendor_gemm"] = _vendor_gemm(torch, wl["hidden"], wl["lm_head"], n, h, v)
 
     if not args.no_cpu_baseline:
         from oracle.cpu_baseline import time_cpu_baseline

@@ -1,12 +1,16 @@
 // mj_grpo.hip -- C ABI (include/mj_grpo.h) and launch plan of the fused GRPO loss path.
 #include "../../include/mj_grpo.h"
+#include "../../include/mj_norm.h"
 
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <initializer_list>
+
 #include "mj_grpo_kernels.hpp"
+#include "mj_norm_kernels.hpp"
 
 namespace {
 
@@ -349,6 +353,83 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
                      size_t workspace_bytes, void* stream) {
   return run(kBackwardOnly, desc, hidden, lm_head, targets, old_logp, advantages, mask, nullptr, nullptr,
              nullptr, nullptr, lse, logp, d_hidden, d_lm_head, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"
+
+// ----------------------------------------------------------------------------- RMSNorm
+namespace {
+constexpr int kNormMaxH = 8192;
+int norm_grid(int64_t n) {   // workgroups of the backward: enough to fill the GPU, each walks rows with this stride
+  const int64_t blocks = (n + 3) / 4;
+  return (int)(blocks < 1024 ? blocks : 1024);
+}
+int norm_check(int64_t n, int64_t h, std::initializer_list<int64_t> lds, std::initializer_list<const void*> ptrs) {
+  if (n <= 0 || h <= 0 || n > (1ll << 30)) return fail(MJ_GRPO_ERR_SHAPE, "rmsnorm: n and h must be positive (got %lld, %lld)", (long long)n, (long long)h);
+  if (h % 8 || h > kNormMaxH) return fail(h % 8 ? MJ_GRPO_ERR_ALIGN : MJ_GRPO_ERR_UNSUPPORTED, "rmsnorm: h must be a multiple of 8 and <= %d (got %lld)", kNormMaxH, (long long)h);
+  for (int64_t ld : lds) {
+    if (ld < h) return fail(MJ_GRPO_ERR_SHAPE, "rmsnorm: leading dimension smaller than h");
+    if (ld % 8) return fail(MJ_GRPO_ERR_ALIGN, "rmsnorm: leading dimensions must be multiples of 8");
+  }
+  for (const void* q : ptrs) {
+    if (q == nullptr) return fail(MJ_GRPO_ERR_NULL, "rmsnorm: NULL pointer argument");
+    if (misaligned(q)) return fail(MJ_GRPO_ERR_ALIGN, "rmsnorm: pointers must be 16-byte aligned");
+  }
+  return MJ_GRPO_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int mj_rmsnorm_forward(const void* x, int64_t ld_x, const float* scale, void* y, int64_t ld_y, float* rstd,
+                       int64_t n, int64_t h, float eps, void* stream) {
+  int rc = norm_check(n, h, {ld_x, ld_y}, {x, scale, y});
+  if (rc) return rc;
+  mj::NormFwdArgs a;
+  a.x = (const uint16_t*)x; a.scale = scale; a.y = (uint16_t*)y; a.rstd = rstd;
+  a.ld_x = ld_x; a.ld_y = ld_y; a.n = (int)n; a.H = (int)h; a.eps = eps;
+  const unsigned grid = (unsigned)((n + 3) / 4);
+  if (h <= 4096) mj::k_rmsnorm_fwd<8><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+  else mj::k_rmsnorm_fwd<16><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+  return check_launch("k_rmsnorm_fwd");
+}
+
+int mj_rmsnorm_workspace_bytes(int64_t n, int64_t h, size_t* bytes) {
+  int rc = norm_check(n, h, {}, {});
+  if (rc) return rc;
+  if (bytes) *bytes = (size_t)norm_grid(n) * (size_t)h * 4;
+  return MJ_GRPO_OK;
+}
+
+int mj_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x, int64_t ld_x, const float* scale, void* dx,
+                        int64_t ld_dx, float* dscale, int accumulate_dscale, int64_t n, int64_t h, float eps,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = norm_check(n, h, {ld_dy, ld_x, ld_dx}, {dy, x, scale, dx, workspace});
+  if (rc) return rc;
+  if (dscale == nullptr) return fail(MJ_GRPO_ERR_NULL, "rmsnorm: dscale is NULL");
+  const int grid = norm_grid(n);
+  const size_t need = (size_t)grid * (size_t)h * 4;
+  if (workspace_bytes < need) return fail(MJ_GRPO_ERR_WORKSPACE, "rmsnorm: workspace too small: %zu < %zu bytes", workspace_bytes, need);
+  mj::NormBwdArgs a;
+  a.dy = (const uint16_t*)dy; a.x = (const uint16_t*)x; a.scale = scale; a.dx = (uint16_t*)dx;
+  a.part = (float*)workspace; a.ld_dy = ld_dy; a.ld_x = ld_x; a.ld_dx = ld_dx; a.n = (int)n; a.H = (int)h; a.eps = eps;
+  const size_t lds = 3 * (size_t)h * 4;
+  hipStream_t st = (hipStream_t)stream;
+  if (h <= 4096) {
+    mj::k_rmsnorm_bwd<8><<<grid, 256, lds, st>>>(a);
+  } else {
+    static thread_local bool raised = false;
+    if (!raised) {
+      hipError_t e = hipFuncSetAttribute((const void*)mj::k_rmsnorm_bwd<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * kNormMaxH * 4);
+      if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+      raised = true;
+    }
+    mj::k_rmsnorm_bwd<16><<<grid, 256, lds, st>>>(a);
+  }
+  if ((rc = check_launch("k_rmsnorm_bwd"))) return rc;
+  mj::k_rmsnorm_dscale<<<(unsigned)((h + 255) / 256), 256, 0, st>>>((const float*)workspace, grid, (int)h, dscale,
+                                                                  accumulate_dscale);
+  return check_launch("k_rmsnorm_dscale");
 }
 
 }  // extern "C"

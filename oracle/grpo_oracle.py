@@ -13,6 +13,7 @@ reference's un-fused jnp loss:
   plugins/training/advantage/grpo.py:28-52     (group-normalised advantages)
   plugins/training/ppo/module.py:59-150        (actor-critic twin: policy + value + entropy bonus)
   plugins/sft/jax/sft_module.py:22-45          (masked cross-entropy)
+  MLLM_JAX/language/llama/llama.py:426-452     (RMSNorm producing `hidden`)
 
 The arithmetic itself lives in un-vendored JAX (jax.nn.log_softmax, jax.nn.softmax,
 jnp.take_along_axis, jnp.clip, jnp.minimum, jax.value_and_grad; version unpinned in
@@ -218,6 +219,24 @@ def ppo_actor_critic_loss(hidden, lm_head, value_w, value_b, target_ids, old_log
         out["d_value_w"] = h.T @ dv
         out["d_value_b"] = dv.sum()
     return out
+
+
+def rms_norm(x, scale, eps=1e-6, dy=None):
+    """LlamaRMSNorm (MLLM_JAX/language/llama/llama.py:438-451), float64:
+    y = x * rsqrt(mean(x^2, -1) + eps) * scale.  With dy, also the transpose
+    (dx, dscale) that jax.value_and_grad yields:
+      gs = dy*scale;  dx = r*gs - x*r^3*mean(gs*x);  dscale = sum_rows dy*x*r."""
+    x = np.asarray(x, np.float64)
+    s = np.asarray(scale, np.float64)
+    r = 1.0 / np.sqrt((x * x).mean(-1, keepdims=True) + float(eps))
+    y = x * r * s
+    if dy is None:
+        return y
+    dy = np.asarray(dy, np.float64)
+    gs = dy * s
+    dx = r * gs - x * r ** 3 * (gs * x).mean(-1, keepdims=True)
+    dscale = (dy * x * r).reshape(-1, x.shape[-1]).sum(0)
+    return y, dx, dscale
 
 
 # --------------------------------------------------------------------------- siblings

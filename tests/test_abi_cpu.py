@@ -29,8 +29,8 @@ def _desc(lib, **kw):
 
 
 def test_header_symbols_are_exported(lib):
-    header = open(os.path.join(ROOT, "include", "mj_grpo.h")).read()
-    declared = set(re.findall(r"\b(mj_grpo_[a-z_]+)\s*\(", header))
+    header = open(os.path.join(ROOT, "include", "mj_grpo.h")).read() + open(os.path.join(ROOT, "include", "mj_norm.h")).read()
+    declared = set(re.findall(r"\b(mj_(?:grpo|rmsnorm)_[a-z_]+)\s*\(", header))
     assert declared == set(lib.EXPORTS)
     handle = lib.load()
     for name in declared:
@@ -109,3 +109,19 @@ def test_workload_generator_shapes_and_advantages():
     wl = make_workload(tiny, "cpu", 1)
     assert wl["hidden"].shape == (512, 16) and wl["lm_head"].shape == (16, 64)
     assert wl["advantages"].abs().max() > 0 and wl["total_valid_token_count"] == wl["mask"].sum().item()
+
+
+def test_rmsnorm_argument_checks_before_any_launch(lib):
+    h = lib.load()
+    fake = 0x1000   # never dereferenced: argument checks fail first
+    sz = C.c_size_t()
+    assert h.mj_rmsnorm_workspace_bytes(4096, 3584, C.byref(sz)) == 0 and sz.value == 1024 * 3584 * 4
+    assert h.mj_rmsnorm_workspace_bytes(10, 64, C.byref(sz)) == 0 and sz.value == 3 * 64 * 4
+    assert h.mj_rmsnorm_workspace_bytes(0, 64, C.byref(sz)) == 2
+    assert h.mj_rmsnorm_workspace_bytes(8, 60, C.byref(sz)) == 3
+    assert h.mj_rmsnorm_workspace_bytes(8, 16384, C.byref(sz)) == 5 and b"8192" in h.mj_grpo_last_error()
+    assert h.mj_rmsnorm_forward(None, 64, fake, fake, 64, None, 8, 64, 1e-6, None) == 1
+    assert h.mj_rmsnorm_forward(fake, 56, fake, fake, 64, None, 8, 64, 1e-6, None) == 2      # ld < h
+    assert h.mj_rmsnorm_forward(fake + 4, 64, fake, fake, 64, None, 8, 64, 1e-6, None) == 3  # alignment
+    assert h.mj_rmsnorm_backward(fake, 64, fake, 64, fake, fake, 64, fake, 0, 8, 64, 1e-6, fake, 16, None) == 4
+    assert b"workspace too small" in h.mj_grpo_last_error()

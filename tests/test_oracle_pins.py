@@ -336,3 +336,28 @@ def test_ppo_uniform_policy_has_maximal_entropy_and_no_entropy_gradient():
                                   entropy_coef=0.5, value_coef=0.0)
     np.testing.assert_allclose(out["entropy"], np.log(v), atol=1e-6)       # 1e-9 inside the log, module.py:76
     np.testing.assert_allclose(out["d_lm_head"], 0.0, atol=1e-15)
+
+
+# --------------------------------------------------------------------------- RMSNorm
+def test_rms_norm_matches_torch_and_autograd(rng):
+    x = rng.standard_normal((5, 24)); s = rng.standard_normal(24); dy = rng.standard_normal((5, 24))
+    xt = torch.tensor(x, requires_grad=True); st = torch.tensor(s, requires_grad=True)
+    yt = torch.nn.functional.rms_norm(xt, (24,), st, eps=1e-6)
+    yt.backward(torch.tensor(dy))
+    y, dx, ds = O.rms_norm(x, s, 1e-6, dy)
+    np.testing.assert_allclose(y, yt.detach().numpy(), rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(dx, xt.grad.numpy(), rtol=1e-10, atol=1e-13)
+    np.testing.assert_allclose(ds, st.grad.numpy(), rtol=1e-10, atol=1e-13)
+
+
+def test_rms_norm_closed_forms():
+    # a constant row c: y = sign(c) * scale / sqrt(1 + eps / c^2); rescaling x leaves y unchanged as eps -> 0
+    s = np.array([1.0, -2.0, 0.5, 3.0])
+    y = O.rms_norm(np.full((1, 4), -3.0), s, 1e-6)
+    np.testing.assert_allclose(y[0], -s / np.sqrt(1 + 1e-6 / 9.0), rtol=1e-14)
+    x = np.array([[1.0, 2.0, -2.0, 4.0]])
+    np.testing.assert_allclose(O.rms_norm(x, s, 0.0), O.rms_norm(7.0 * x, s, 0.0), rtol=1e-14)
+    np.testing.assert_allclose(O.rms_norm(x, s, 0.0)[0], x[0] / 2.5 * s, rtol=1e-14)   # rms = sqrt(25/4)
+    # dx is orthogonal to x when eps = 0 (the norm is scale invariant)
+    _, dx, _ = O.rms_norm(x, s, 0.0, np.array([[0.3, -1.0, 2.0, 0.7]]))
+    assert abs((dx * x).sum()) < 1e-13
