@@ -113,6 +113,14 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
                      const float* mask, const float* lse, const float* logp, void* d_hidden,
                      float* d_lm_head, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Group-normalised advantages on the device: advantages[i] = (r_i - mean_g) / (std_g + eps) over
+ * the samples that share group_ids[i] (population std; any int ids, any group sizes).  Replaces
+ * compute_grpo_advantages_by_group_id (plugins/training/advantage/grpo.py:8-52), which the
+ * runner evaluates in host NumPy (runner/grpo_gsm8k.py:680).  rewards, advantages: float32 [b];
+ * group_ids: int32 [b]. */
+int mj_grpo_group_advantages(const float* rewards, const int32_t* group_ids, float* advantages,
+                             int64_t b, float eps, void* stream);
+
 /* Optional per-kernel timing (bench and profiling; no counterpart in the reference, whose only
  * timers are wall-clock phase timers, plugins/training/runner/grpo_gsm8k.py:615-792).
  * Between begin and end every kernel launch of the entry points above is bracketed by a pair of

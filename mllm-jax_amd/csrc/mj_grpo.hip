@@ -1,6 +1,7 @@
 // mj_grpo.hip -- C ABI (include/mj_grpo.h) and launch plan of the fused GRPO loss path.
 #include "../../include/mj_grpo.h"
 #include "../../include/mj_norm.h"
+#include "../../include/mj_sample.h"
 
 #include <hip/hip_runtime.h>
 #include <math.h>
@@ -81,8 +82,10 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   if (d->n_tokens <= 0 || d->hidden <= 0 || d->vocab <= 0)
     return fail(MJ_GRPO_ERR_SHAPE, "n_tokens/hidden/vocab must be positive (got %lld/%lld/%lld)",
                 (long long)d->n_tokens, (long long)d->hidden, (long long)d->vocab);
-  if (d->n_tokens > (1ll << 30) || d->hidden > (1 << 20) || d->vocab > (1 << 24))
-    return fail(MJ_GRPO_ERR_SHAPE, "shape too large");
+  // 256 rows of any operand or output must fit one 2 GiB buffer descriptor
+  if (d->n_tokens > (1ll << 30) || d->hidden > (1 << 20) || d->vocab > (1 << 21) || d->ld_hidden > (1 << 20) ||
+      d->ld_w > (1 << 21) || d->chunk_tokens > (1 << 20))
+    return fail(MJ_GRPO_ERR_SHAPE, "shape too large (hidden, ld_hidden <= 2^20; vocab, ld_w <= 2^21; chunk_tokens <= 2^20)");
   if (d->ld_hidden < d->hidden || d->ld_w < d->vocab)
     return fail(MJ_GRPO_ERR_SHAPE, "leading dimension smaller than row length");
   if (d->hidden % 8 || d->vocab % 8 || d->ld_hidden % 8 || d->ld_w % 8)
@@ -357,6 +360,56 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
 
 }  // extern "C"
 
+extern "C" int mj_grpo_group_advantages(const float* rewards, const int32_t* group_ids, float* advantages, int64_t b,
+                                        float eps, void* stream) {
+  if (!rewards || !group_ids || !advantages) return fail(MJ_GRPO_ERR_NULL, "rewards/group_ids/advantages is NULL");
+  if (b <= 0 || b > (1 << 20)) return fail(MJ_GRPO_ERR_SHAPE, "batch must be in [1, 2^20] (got %lld)", (long long)b);
+  mj::k_group_advantages<<<(unsigned)((b + 255) / 256), 256, 0, (hipStream_t)stream>>>(rewards, group_ids, advantages,
+                                                                                         (int)b, eps);
+  return check_launch("k_group_advantages");
+}
+
+// ----------------------------------------------------------------------------- sampler
+extern "C" {
+
+int mj_sample_logits(const void* hidden, int64_t ld_hidden, const void* lm_head, int64_t ld_w, float* logits,
+                     int64_t ld_logits, int64_t b, int64_t h, int64_t vocab, float softcap, void* stream) {
+  if (!hidden || !lm_head || !logits) return fail(MJ_GRPO_ERR_NULL, "hidden/lm_head/logits is NULL");
+  if (b <= 0 || h <= 0 || vocab <= 0 || b > (1 << 24) || h > (1 << 20) || vocab > (1 << 21))
+    return fail(MJ_GRPO_ERR_SHAPE, "sample_logits: bad shape b=%lld h=%lld vocab=%lld", (long long)b, (long long)h, (long long)vocab);
+  if (ld_hidden < h || ld_w < vocab || ld_logits < vocab) return fail(MJ_GRPO_ERR_SHAPE, "sample_logits: leading dimension smaller than row length");
+  if (h % 8 || vocab % 8 || ld_hidden % 8 || ld_w % 8 || ld_logits % 4)
+    return fail(MJ_GRPO_ERR_ALIGN, "sample_logits: h, vocab, ld_hidden, ld_w must be multiples of 8 and ld_logits of 4");
+  if (misaligned(hidden) || misaligned(lm_head) || misaligned(logits)) return fail(MJ_GRPO_ERR_ALIGN, "sample_logits: pointers must be 16-byte aligned");
+  if (!(softcap >= 0.f) || !isfinite(softcap)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "sample_logits: softcap must be >= 0");
+  if (ld_w > (1 << 21) || ld_logits > (1 << 21) || ld_hidden > (1 << 20))
+    return fail(MJ_GRPO_ERR_SHAPE, "sample_logits: leading dimensions too large (ld_hidden <= 2^20; ld_w, ld_logits <= 2^21)");
+  int rc;
+  if ((rc = enable_lds(mj::k_logits_rows<BM, BN>))) return rc;
+  mj::LogitsRowsArgs a;
+  a.w = (const __bf16*)lm_head; a.hid = (const __bf16*)hidden; a.ld_w = ld_w; a.ld_hid = ld_hidden;
+  a.V = (int)vocab; a.n = (int)b; a.H = (int)h; a.cap = softcap; a.out = logits; a.ld_out = ld_logits;
+  const mj::TileMap map((int)((vocab + BM - 1) / BM), (int)((b + BN - 1) / BN), 1);
+  mj::k_logits_rows<BM, BN><<<map.items(), mj::kThreads, mj::GemmTN<BM, BN>::kLdsBytes, (hipStream_t)stream>>>(a, map);
+  return check_launch("k_logits_rows");
+}
+
+int mj_sample_top_k(const float* logits, int64_t ld_logits, int64_t b, int64_t vocab, int k, float temperature,
+                    const float* noise, int32_t* token, int32_t* top_idx, float* top_val, void* stream) {
+  if (!logits || !token) return fail(MJ_GRPO_ERR_NULL, "sample_top_k: logits/token is NULL");
+  if (b <= 0 || vocab <= 0 || b > (1 << 24) || vocab > (1 << 30) || ld_logits < vocab)
+    return fail(MJ_GRPO_ERR_SHAPE, "sample_top_k: bad shape b=%lld vocab=%lld ld=%lld", (long long)b, (long long)vocab, (long long)ld_logits);
+  if (k < 1 || k > mj::kTopKMax || k > vocab) return fail(MJ_GRPO_ERR_UNSUPPORTED, "sample_top_k: k must be in [1, min(%d, vocab)] (got %d)", mj::kTopKMax, k);
+  if (!(temperature > 0.f) || !isfinite(temperature)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "sample_top_k: temperature must be > 0");
+  mj::TopKArgs a;
+  a.logits = logits; a.ld = ld_logits; a.V = (int)vocab; a.k = k; a.inv_t = 1.f / temperature; a.noise = noise;
+  a.token = token; a.top_idx = top_idx; a.top_val = top_val;
+  mj::k_topk_sample<<<(unsigned)b, 1024, 0, (hipStream_t)stream>>>(a);
+  return check_launch("k_topk_sample");
+}
+
+}  // extern "C"
+
 // ----------------------------------------------------------------------------- RMSNorm
 namespace {
 constexpr int kNormMaxH = 8192;
@@ -438,3 +491,4 @@ int mj_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x, int64_t ld
 template __global__ void mj::k_logits_stats<256, 256>(mj::LogitsArgs, mj::TileMap);
 template __global__ void mj::k_dhidden<256, 256>(mj::DhArgs, mj::TileMap);
 template __global__ void mj::k_dw<256, 256>(mj::DwArgs, mj::TileMap);
+template __global__ void mj::k_logits_rows<256, 256>(mj::LogitsRowsArgs, mj::TileMap);

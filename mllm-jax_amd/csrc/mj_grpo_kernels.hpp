@@ -492,4 +492,201 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
   }
 }
 
+// ----------------------------------------------------------------------------- sampling
+// Last-position logits for the sampler, float32 row-major [n, ld_out]: same product as
+// k_logits_stats (W read in place as the row operand), plain store epilogue -- a lane's four
+// consecutive accumulator rows are four consecutive vocab entries of its token's row.
+struct LogitsRowsArgs {
+  const __bf16* w;       // lm_head [H, ld_w]
+  const __bf16* hid;     // [n, ld_hid]
+  int64_t ld_w, ld_hid;
+  int V, n, H;
+  float cap;             // final-logit softcap, 0 = off
+  float* out;            // [n, ld_out]
+  int64_t ld_out;
+};
+
+template <int BM, int BN>
+__global__ __launch_bounds__(kThreads) void k_logits_rows(LogitsRowsArgs p, TileMap map) {
+  using G = GemmTN<BM, BN, kKRow, kRowK>;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  int tm, tn, split;
+  if (!map.tile(blockIdx.x, tm, tn, split)) return;
+  const int m0 = tm * BM, n0 = tn * BN;
+  G g;
+  g.run(p.w + m0, p.V - m0, p.ld_w, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0, p.ld_hid, p.H, smem);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
+  const int t0 = n0 + wn * G::WN, v0 = m0 + wm * G::WM;
+  const int trows = min(max(p.n - t0, 0), G::WN);
+  const uint32_t ld4 = (uint32_t)p.ld_out * 4;
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc_wave(p.out + (int64_t)t0 * p.ld_out + v0, (int64_t)trows * ld4 - (int64_t)v0 * 4);
+  const int vleft = p.V - v0;
+  const float inv_cap = p.cap > 0.f ? 1.f / p.cap : 0.f;
+#pragma unroll
+  for (int ni = 0; ni < G::NI; ++ni) {
+    const uint32_t lane_off = (uint32_t)((ni * 32 + l31) * ld4 + lhi * 16);
+#pragma unroll
+    for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int vv = mi * 32 + q * 8;
+        const uint32_t voff = (vv + lhi * 4) < vleft ? lane_off : kOob;
+        f32x4 a = {g.acc[mi][ni][q * 4], g.acc[mi][ni][q * 4 + 1], g.acc[mi][ni][q * 4 + 2], g.acc[mi][ni][q * 4 + 3]};
+        if (p.cap > 0.f) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) a[j] = softcap_apply(a[j], p.cap, inv_cap);
+        }
+        store_b128(a, rs, voff, (uint32_t)vv * 4);
+      }
+  }
+}
+
+// Top-k + categorical draw per row (MLLM_JAX/sample/sanple_utils.py:35-53): the k largest of
+// logits / t (ties: lower index first, like jax.lax.top_k), then argmax_j(top_j + noise_j) where
+// noise holds the caller's Gumbel samples -- what jax.random.categorical evaluates.  One
+// workgroup per row: an 8-bit-per-pass radix select over order-preserving keys finds the k-th
+// largest key, elements above it are collected in any order, elements equal to it in index order.
+constexpr int kTopKMax = 64;
+struct TopKArgs {
+  const float* logits;   // [b, ld]
+  int64_t ld;
+  int V, k;
+  float inv_t;
+  const float* noise;    // [b, k] or null (greedy: the largest)
+  int32_t* token;        // [b]
+  int32_t* top_idx;      // [b, k] or null
+  float* top_val;        // [b, k] or null (logits / t, descending)
+};
+
+MJ_DEV uint32_t topk_key(float f) {   // larger float <=> larger key; -0 and +0 differ only in sign bit order
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t s_prefix, s_need, s_cnt, s_wave[16], s_base;
+  __shared__ float c_val[kTopKMax], o_val[kTopKMax];
+  __shared__ int c_idx[kTopKMax], o_idx[kTopKMax];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const float* row = p.logits + (int64_t)blockIdx.x * p.ld;
+  // the k-th largest key, most significant byte first
+  uint32_t prefix = 0, need = (uint32_t)p.k;   // `need` keys still to find among those matching `prefix`
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    if (tid < 256) hist[tid] = 0;
+    __syncthreads();
+    const uint32_t hi_mask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
+    for (int i = tid; i < p.V; i += 1024) {
+      const uint32_t key = topk_key(row[i] * p.inv_t);
+      if ((key & hi_mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    if (tid == 0) {
+      uint32_t acc = 0;
+      int bin = 255;
+      for (; bin > 0; --bin) {
+        if (acc + hist[bin] >= need) break;
+        acc += hist[bin];
+      }
+      s_prefix = prefix | ((uint32_t)bin << shift);
+      s_need = need - acc;
+    }
+    __syncthreads();
+    prefix = s_prefix;
+    need = s_need;
+    __syncthreads();
+  }
+  // prefix = key of the k-th largest; `need` of the elements equal to it belong to the top k
+  if (tid == 0) { s_cnt = 0; s_base = 0; }
+  __syncthreads();
+  for (int i = tid; i < p.V; i += 1024) {
+    const float v = row[i] * p.inv_t;
+    if (topk_key(v) > prefix) {
+      const uint32_t slot = atomicAdd(&s_cnt, 1u);
+      c_val[slot] = v;
+      c_idx[slot] = i;
+    }
+  }
+  __syncthreads();
+  const uint32_t above = s_cnt;            // == k - need
+  // equal keys in index order: block-wide ranks, 1024 elements at a time, until `need` are taken
+  for (int i0 = 0; i0 < p.V; i0 += 1024) {
+    if (s_base >= need) break;             // uniform: s_base is read after the barrier below
+    const int i = i0 + tid;
+    const float v = i < p.V ? row[i] * p.inv_t : 0.f;
+    const bool eq = i < p.V && topk_key(v) == prefix;
+    const unsigned long long m = __ballot(eq);
+    if (lane == 0) s_wave[wave] = (uint32_t)__popcll(m);
+    __syncthreads();
+    uint32_t before = s_base;
+    for (int w = 0; w < wave; ++w) before += s_wave[w];
+    const uint32_t rank = before + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+    if (eq && rank < need) {
+      c_val[above + rank] = v;
+      c_idx[above + rank] = i;
+    }
+    __syncthreads();
+    if (tid == 0) {
+      uint32_t t = s_base;
+      for (int w = 0; w < 16; ++w) t += s_wave[w];
+      s_base = t;
+    }
+    __syncthreads();
+  }
+  // order the k candidates: value descending, index ascending
+  if (tid < p.k) {
+    const float v = c_val[tid];
+    const int ix = c_idx[tid];
+    int r = 0;
+    for (int j = 0; j < p.k; ++j) {
+      const float vj = c_val[j];
+      r += (vj > v || (vj == v && c_idx[j] < ix)) ? 1 : 0;
+    }
+    o_val[r] = v;
+    o_idx[r] = ix;
+  }
+  __syncthreads();
+  if (tid < p.k) {
+    if (p.top_idx != nullptr) p.top_idx[(int64_t)blockIdx.x * p.k + tid] = o_idx[tid];
+    if (p.top_val != nullptr) p.top_val[(int64_t)blockIdx.x * p.k + tid] = o_val[tid];
+  }
+  if (tid == 0) {
+    int best = 0;
+    if (p.noise != nullptr) {
+      float bs = o_val[0] + p.noise[(int64_t)blockIdx.x * p.k];
+      for (int j = 1; j < p.k; ++j) {
+        const float sc = o_val[j] + p.noise[(int64_t)blockIdx.x * p.k + j];
+        if (sc > bs) { bs = sc; best = j; }      // first maximum wins, like argmax
+      }
+    }
+    p.token[blockIdx.x] = o_idx[best];
+  }
+}
+
+// ----------------------------------------------------------------------------- advantages
+// Group-normalised advantages (plugins/training/advantage/grpo.py:28-52): per group id,
+// (r - mean) / (std + eps) with the population std.  B is a batch of sequences (hundreds), so
+// each thread simply walks the batch for its own element: sums in double in index order (what
+// np.bincount does), the remaining arithmetic in float like the NumPy original.
+__global__ __launch_bounds__(256) void k_group_advantages(const float* rewards, const int32_t* group_ids, float* adv,
+                                                          int b, float eps) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= b) return;
+  const int gid = group_ids[i];
+  double sum = 0.0;
+  int cnt = 0;
+  for (int j = 0; j < b; ++j)
+    if (group_ids[j] == gid) { sum += (double)rewards[j]; ++cnt; }
+  const float count = fmaxf((float)cnt, 1.f);
+  const float mean = (float)sum / count;
+  double sq = 0.0;
+  for (int j = 0; j < b; ++j)
+    if (group_ids[j] == gid) { const float c = rewards[j] - mean; sq += (double)(c * c); }
+  const float var = (float)sq / count;
+  adv[i] = (rewards[i] - mean) / (sqrtf(var) + eps);
+}
+
 }  // namespace mj

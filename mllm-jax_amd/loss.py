@@ -424,6 +424,30 @@ class PPOActorCriticModule:
                 "per_token_logps": p.logp.reshape(b, t)}
 
 
+def compute_grpo_advantages_by_group_id(*, rewards, group_ids, eps: float = 1e-4) -> torch.Tensor:
+    """Device counterpart of plugins/training/advantage/grpo.py:8-52: float32 advantages [B],
+    (r - mean_g) / (std_g + eps) within each group id (population std, variable group sizes).
+    `rewards` must be a GPU tensor; `group_ids` is moved beside it."""
+    rewards = torch.as_tensor(rewards)
+    if rewards.device.type != "cuda":
+        raise RuntimeError("compute_grpo_advantages_by_group_id needs GPU tensors; there is no CPU path")
+    if rewards.dim() != 1:
+        raise ValueError(f"rewards must be rank-1 [B], got shape={tuple(rewards.shape)}")
+    group_ids = torch.as_tensor(group_ids, device=rewards.device)
+    if group_ids.shape != rewards.shape:
+        raise ValueError(f"group_ids must have same shape as rewards, got {tuple(group_ids.shape)} vs "
+                         f"{tuple(rewards.shape)}")
+    if rewards.numel() == 0:
+        raise ValueError("No groups found (empty batch?)")
+    r = rewards.to(torch.float32).contiguous()
+    g = group_ids.to(torch.int32).contiguous()
+    out = torch.empty_like(r)
+    with torch.cuda.device(r.device):
+        _lib.check(_lib.load().mj_grpo_group_advantages(r.data_ptr(), g.data_ptr(), out.data_ptr(), r.numel(),
+                                                        float(eps), torch.cuda.current_stream(r.device).cuda_stream))
+    return out
+
+
 def loss_and_metrics(module: Callable[[Mapping[str, Any]], dict], inputs: Mapping[str, Any]):
     """loss_fn of plugins/training/update/train_step.py:15-22: pops per_token_logps, means
     the other metrics, returns (loss, metrics | {"per_token_logps": ...})."""

@@ -14,6 +14,7 @@ reference's un-fused jnp loss:
   plugins/training/ppo/module.py:59-150        (actor-critic twin: policy + value + entropy bonus)
   plugins/sft/jax/sft_module.py:22-45          (masked cross-entropy)
   MLLM_JAX/language/llama/llama.py:426-452     (RMSNorm producing `hidden`)
+  MLLM_JAX/sample/sanple_utils.py:35-60        (top-k / categorical draw of the sampler)
 
 The arithmetic itself lives in un-vendored JAX (jax.nn.log_softmax, jax.nn.softmax,
 jnp.take_along_axis, jnp.clip, jnp.minimum, jax.value_and_grad; version unpinned in
@@ -25,6 +26,9 @@ the six clip regions enumerated by hand, torch.autograd in float64 and central
 finite differences for the backward, softcap limits, permutation invariance.
 
 Parity unpinned (documented, accepted):
+  * jax.random's threefry stream behind jax.random.categorical: the draw is restated as
+    argmax(x + Gumbel noise) with the noise an input; which token a given JAX key yields is
+    not reproduced.
   * XLA's bf16 rounding of logits under the Qwen dtype policy
     (modular_qwen2.py:143, llama.py:255-256) is deliberately not replicated: the
     oracle keeps float64 logits of bf16-valued inputs.
@@ -237,6 +241,23 @@ def rms_norm(x, scale, eps=1e-6, dy=None):
     dx = r * gs - x * r ** 3 * (gs * x).mean(-1, keepdims=True)
     dscale = (dy * x * r).reshape(-1, x.shape[-1]).sum(0)
     return y, dx, dscale
+
+
+def top_k_sample(logits, k=50, t=0.9, noise=None):
+    """_top_k_sampling_batched (MLLM_JAX/sample/sanple_utils.py:35-53) with the categorical draw
+    written as argmax(top_logits + Gumbel noise) (what jax.random.categorical evaluates).
+    logits [B,V] float32; scaled = logits * float32(1/t) in float32; top-k in descending order,
+    equal values by ascending index (jax.lax.top_k); noise [B,k] or None (greedy).
+    Returns (token[B], top_idx[B,k], top_val[B,k])."""
+    x = np.asarray(logits, np.float32) * np.float32(1.0 / float(t))
+    b, v = x.shape
+    order = np.lexsort((np.broadcast_to(np.arange(v), x.shape), -x.astype(np.float64)), axis=-1)[:, :k]
+    top_val = np.take_along_axis(x, order, axis=-1)
+    if noise is None:
+        pick = np.zeros(b, np.int64)
+    else:
+        pick = np.argmax(top_val + np.asarray(noise, np.float32), axis=-1)      # first maximum
+    return order[np.arange(b), pick].astype(np.int32), order.astype(np.int32), top_val
 
 
 # --------------------------------------------------------------------------- siblings

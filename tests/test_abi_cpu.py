@@ -29,8 +29,9 @@ def _desc(lib, **kw):
 
 
 def test_header_symbols_are_exported(lib):
-    header = open(os.path.join(ROOT, "include", "mj_grpo.h")).read() + open(os.path.join(ROOT, "include", "mj_norm.h")).read()
-    declared = set(re.findall(r"\b(mj_(?:grpo|rmsnorm)_[a-z_]+)\s*\(", header))
+    header = open(os.path.join(ROOT, "include", "mj_grpo.h")).read() + open(os.path.join(ROOT, "include", "mj_norm.h")).read() \
+        + open(os.path.join(ROOT, "include", "mj_sample.h")).read()
+    declared = set(re.findall(r"\b(mj_(?:grpo|rmsnorm|sample)_[a-z_]+)\s*\(", header))
     assert declared == set(lib.EXPORTS)
     handle = lib.load()
     for name in declared:
@@ -125,3 +126,16 @@ def test_rmsnorm_argument_checks_before_any_launch(lib):
     assert h.mj_rmsnorm_forward(fake + 4, 64, fake, fake, 64, None, 8, 64, 1e-6, None) == 3  # alignment
     assert h.mj_rmsnorm_backward(fake, 64, fake, 64, fake, fake, 64, fake, 0, 8, 64, 1e-6, fake, 16, None) == 4
     assert b"workspace too small" in h.mj_grpo_last_error()
+
+
+def test_sampler_argument_checks_before_any_launch(lib):
+    h = lib.load()
+    fake = 0x1000
+    assert h.mj_sample_logits(None, 64, fake, 512, fake, 512, 4, 64, 512, 0.0, None) == 1
+    assert h.mj_sample_logits(fake, 64, fake, 512, fake, 500, 4, 64, 512, 0.0, None) == 2
+    assert h.mj_sample_logits(fake, 64, fake, 516, fake, 520, 4, 64, 516, 0.0, None) == 3
+    assert h.mj_sample_logits(fake, 64, fake, 512, fake, 512, 4, 64, 512, -1.0, None) == 5
+    assert h.mj_sample_top_k(fake, 512, 4, 512, 65, 1.0, None, fake, None, None, None) == 5
+    assert h.mj_sample_top_k(fake, 512, 4, 40, 50, 1.0, None, fake, None, None, None) == 5      # k > vocab
+    assert h.mj_sample_top_k(fake, 512, 4, 512, 50, 0.0, None, fake, None, None, None) == 5
+    assert h.mj_sample_top_k(fake, 512, 4, 512, 50, 1.0, None, None, None, None, None) == 1

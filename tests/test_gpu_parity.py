@@ -260,3 +260,26 @@ def test_error_paths_on_device():
         M.grpo_fused_loss(hid.to(d), w[:, :291].contiguous().to(d), y.to(d) % 291, None, adv.to(d), mask.to(d))
     with pytest.raises(RuntimeError):   # CPU tensors: no fallback
         M.grpo_fused_loss(hid, w, y, None, adv, mask)
+
+
+def test_group_advantages_on_device():
+    import mllm_jax_amd as M
+    d = _dev()
+    # the reference's own known answers for this estimator's siblings use this batch
+    # (tests/test_advantage_estimators.py:33-34); the closed form is written out here
+    r = np.asarray([1.0, 2.0, 3.0, 10.0, 20.0], np.float32); gid = np.asarray([0, 0, 0, 1, 1], np.int32)
+    out = M.compute_grpo_advantages_by_group_id(rewards=torch.tensor(r, device=d), group_ids=torch.tensor(gid), eps=1e-4)
+    s0, s1 = np.sqrt(2.0 / 3.0), 5.0
+    expect = np.array([-1 / (s0 + 1e-4), 0.0, 1 / (s0 + 1e-4), -5 / (s1 + 1e-4), 5 / (s1 + 1e-4)])
+    np.testing.assert_allclose(out.cpu().numpy(), expect, rtol=2e-7, atol=1e-7)
+    # ragged groups, non-contiguous ids, a singleton group, against the oracle
+    rng = np.random.default_rng(4)
+    b = 777
+    gid = rng.choice(np.array([-5, 3, 3000, 17, 42, 99999]), size=b).astype(np.int32)
+    gid[0] = 123456                                      # singleton: advantage 0
+    r = rng.standard_normal(b).astype(np.float32)
+    out = M.compute_grpo_advantages_by_group_id(rewards=torch.tensor(r, device=d), group_ids=torch.tensor(gid, device=d))
+    np.testing.assert_allclose(out.cpu().numpy(), O.grpo_advantages(r, gid), rtol=1e-6, atol=1e-6)
+    assert out[0].item() == 0.0 and out.dtype == torch.float32
+    with pytest.raises(ValueError):
+        M.compute_grpo_advantages_by_group_id(rewards=torch.zeros(4, device=d), group_ids=torch.zeros(3))

@@ -1,0 +1,78 @@
+"""GPU parity of the sampler step: last-position logits against a float64 product, the top-k /
+categorical draw bit-exactly against the CPU oracle on the SAME float32 logits and noise."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import grpo_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def test_last_position_logits_match_float64_product():
+    import mllm_jax_amd as M
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(1)
+    for b, h, v, cap in [(5, 64, 1000, None), (128, 896, 5000, None), (300, 136, 2008, 30.0), (1, 8, 8, None)]:
+        hid = torch.randn(b, h, generator=g).to(torch.bfloat16)
+        w = (0.2 * torch.randn(h, v, generator=g)).to(torch.bfloat16)
+        out = M.last_position_logits(hid.to(dev), w.to(dev), cap)
+        ref = O.lm_head_logits(hid.float().numpy(), w.float().numpy(), cap)
+        assert out.dtype == torch.float32 and tuple(out.shape) == (b, v)
+        np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("b,v,k,t", [(3, 1000, 50, 0.9), (64, 152064, 50, 1.0), (7, 129, 64, 0.7), (2, 50, 50, 1.0),
+                                     (5, 4097, 1, 1.0)])
+def test_top_k_draw_is_bit_exact(b, v, k, t):
+    import mllm_jax_amd as M
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(b * 1000 + k)
+    logits = (3.0 * torch.randn(b, v, generator=g)).float()
+    u = torch.rand(b, k, generator=g)
+    noise = -torch.log(-torch.log(u))
+    tok, idx, val = M.top_k_sampling_batched(noise.to(dev), logits.to(dev), k=k, t=t, return_top_k=True)
+    rt, ri, rv = O.top_k_sample(logits.numpy(), k=k, t=t, noise=noise.numpy())
+    np.testing.assert_array_equal(idx.cpu().numpy(), ri)
+    np.testing.assert_array_equal(val.cpu().numpy(), rv)
+    np.testing.assert_array_equal(tok.cpu().numpy(), rt)
+
+
+def test_ties_duplicates_and_negative_values():
+    import mllm_jax_amd as M
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(0)
+    # few distinct values: the k-th largest is shared by many entries, lower indices must win
+    x = rng.integers(-3, 4, size=(9, 3000)).astype(np.float32)
+    x[4] = -7.0                                             # a constant row: indices 0..k-1
+    x[5, 100:] = -np.inf
+    noise = rng.gumbel(size=(9, 50)).astype(np.float32)
+    tok, idx, val = M.top_k_sampling_batched(torch.tensor(noise), torch.tensor(x, device=dev), k=50, t=1.0, return_top_k=True)
+    rt, ri, rv = O.top_k_sample(x, k=50, t=1.0, noise=noise)
+    np.testing.assert_array_equal(idx.cpu().numpy(), ri)
+    np.testing.assert_array_equal(val.cpu().numpy(), rv)
+    np.testing.assert_array_equal(tok.cpu().numpy(), rt)
+    np.testing.assert_array_equal(idx[4].cpu().numpy(), np.arange(50))
+
+
+def test_greedy_generator_draws_and_fused_step():
+    import mllm_jax_amd as M
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(5)
+    b, h, v = 32, 64, 4000
+    hid = torch.randn(b, h, generator=g).to(torch.bfloat16).to(dev)
+    w = (0.5 * torch.randn(h, v, generator=g)).to(torch.bfloat16).to(dev)
+    logits = M.last_position_logits(hid, w)
+    np.testing.assert_array_equal(M.greedy_sampling(None, logits).cpu().numpy(), logits.argmax(-1).cpu().numpy())
+    gen = torch.Generator(device=dev).manual_seed(7)
+    a = M.sample_next_tokens(gen, hid, w, k=50, t=1.0)
+    gen.manual_seed(7)
+    b2 = M.sample_next_tokens(gen, hid, w, k=50, t=1.0)
+    assert torch.equal(a, b2) and a.dtype == torch.int32               # same generator state, same draw
+    top = torch.topk(logits, 50, dim=-1).indices
+    assert bool((top == a[:, None]).any(-1).all())                      # every draw lies inside its row's top 50
+    # draws follow softmax over the top k: a sharply peaked row is (almost) always its argmax
+    peaked = torch.zeros(1, v, device=dev); peaked[0, 123] = 40.0
+    assert int(M.top_k_sampling_batched(gen, peaked, k=50, t=1.0)[0]) == 123
+    with pytest.raises(M._lib.MjGrpoError):
+        M.top_k_sampling_batched(None, logits, k=65)

@@ -361,3 +361,25 @@ def test_rms_norm_closed_forms():
     # dx is orthogonal to x when eps = 0 (the norm is scale invariant)
     _, dx, _ = O.rms_norm(x, s, 0.0, np.array([[0.3, -1.0, 2.0, 0.7]]))
     assert abs((dx * x).sum()) < 1e-13
+
+
+# --------------------------------------------------------------------------- sampler
+def test_top_k_sample_against_torch_topk_and_by_hand(rng):
+    x = rng.standard_normal((6, 500)).astype(np.float32)
+    tok, idx, val = O.top_k_sample(x, k=7, t=0.5, noise=None)
+    tv, ti = torch.topk(torch.tensor(x) * np.float32(2.0), 7, dim=-1)            # distinct values: order is unique
+    np.testing.assert_array_equal(idx, ti.numpy())
+    np.testing.assert_array_equal(val, tv.numpy())
+    np.testing.assert_array_equal(tok, x.argmax(-1))                             # greedy = the largest
+    # ties go to the lower index; the noise decides among the k
+    y = np.array([[1.0, 3.0, 3.0, 0.0, 3.0, 2.0]], np.float32)
+    tok, idx, val = O.top_k_sample(y, k=4, t=1.0, noise=np.array([[0.0, 0.0, 5.0, 0.0]], np.float32))
+    np.testing.assert_array_equal(idx, [[1, 2, 4, 5]])
+    np.testing.assert_array_equal(val, [[3.0, 3.0, 3.0, 2.0]])
+    assert tok[0] == 4
+    # Gumbel-max over the top k follows softmax(top_logits): frequencies of a 3-way draw
+    z = np.array([[np.log(0.6), np.log(0.3), np.log(0.1), -50.0]], np.float32)
+    u = rng.random((20000, 3)); g = -np.log(-np.log(u))
+    draws = np.array([O.top_k_sample(z, k=3, t=1.0, noise=g[i:i + 1])[0][0] for i in range(0, 20000, 10)])
+    freq = np.bincount(draws, minlength=3) / len(draws)
+    np.testing.assert_allclose(freq, [0.6, 0.3, 0.1], atol=0.04)
