@@ -24,10 +24,10 @@ PEAK_HBM_GBS = 8000.0
 # two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for
 # a plain 1 GiB device copy (x2.00 fetch, x1.00 write); summary in profiles/.  Keyed by
 # (config index, kernel); None for workloads that were not counted.
-MEASURED_TRAFFIC_BYTES = {
-    (2, "k_logits_stats"): 16.78e9,
-    (2, "k_dhidden"): 21.80e9,
-    (2, "k_dw"): 17.41e9,
+MEASURED_TRAFFIC_BYTES = {          # default chunk (16384 tokens: one launch of each kernel per step)
+    (2, "k_logits_stats"): 32.57e9,
+    (2, "k_dhidden"): 51.75e9,
+    (2, "k_dw"): 30.53e9,
 }
 
 
@@ -141,7 +141,7 @@ def main() -> int:
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                 "avg_launch_ms": round(avg_launch_ms, 3), "launches": dom_launches,
                 "flop_per_launch": flop_per_launch,
-                "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom))}
+                "traffic": None if args.chunk_tokens else MEASURED_TRAFFIC_BYTES.get((args.config, dom))}
 
     line = {
         "metric": "grpo_fused_loss_fwd_bwd_tokens_per_s", "value": round(tokens_per_s, 1), "unit": "tokens/s",

@@ -56,7 +56,7 @@ constexpr int64_t kDefaultChunk = 16384;   // tokens whose logits live in the wo
 inline int64_t rup(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 
 struct Plan {
-  int64_t N, H, V, chunk, n_pad, parts;
+  int64_t N, H, V, chunk, n_pad, ld_z, parts;
   int dh_splits;          // vocab splits of the dHidden product (1 = none)
   int64_t dh_k_per_split;
   // byte offsets into the workspace
@@ -103,6 +103,7 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   if (chunk > p->N) chunk = p->N;
   p->chunk = chunk;
   p->n_pad = rup(chunk, 256);
+  p->ld_z = p->n_pad;
   p->parts = 2 * ((p->V + BM - 1) / BM);
   p->dh_splits = pick_splits((p->n_pad / BM) * ((p->H + BN - 1) / BN));
   p->dh_k_per_split = rup((p->V + p->dh_splits - 1) / p->dh_splits, 64);
@@ -118,7 +119,7 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   p->ge = take((size_t)p->n_pad * 4);
   p->hent = take((size_t)p->n_pad * 4);
   p->total_fwd = o;
-  p->zt = take((size_t)p->V * p->n_pad * 2);
+  p->zt = take((size_t)p->V * p->ld_z * 2);
   p->part = take(p->dh_splits > 1 ? (size_t)p->dh_splits * p->n_pad * p->H * 4 : 0);
   p->total_bwd = o;
   return MJ_GRPO_OK;
@@ -200,7 +201,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       mj::LogitsArgs a;
       a.w = (const __bf16*)lm_head; a.hid = hid_c; a.ld_w = d->ld_w; a.ld_hid = d->ld_hidden;
       a.V = V; a.n = nc; a.H = H; a.cap = d->softcap;
-      a.zt = bwd ? zt : nullptr; a.ld_z = p.n_pad;
+      a.zt = bwd ? zt : nullptr; a.ld_z = p.ld_z;
       a.pm = pm; a.pl = pl; a.ps = ps; a.ld_p = p.n_pad;
       a.targets = targets + c0; a.zy = zy + c0;
       const mj::TileMap map((V + BM - 1) / BM, (nc + BN - 1) / BN, 1);
@@ -229,7 +230,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     }
     if (bwd) {
       mj::DzArgs z;
-      z.zt = zt; z.ld_z = p.n_pad;
+      z.zt = zt; z.ld_z = p.ld_z;
       z.lse = (mode == kBackwardOnly ? saved_lse : lse) + c0; z.g = g; z.targets = targets + c0;
       z.ge = bonus ? ge : nullptr; z.hent = bonus ? hent : nullptr;
       z.V = V; z.n = nc; z.n_pad = n_pad; z.cap = d->softcap;
@@ -241,7 +242,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       // the split count was planned for a full chunk; a shorter last chunk keeps it (the partial
       // buffer is sized for it) unless it has a single split anyway
       mj::DhArgs h;
-      h.dzt = (const __bf16*)zt; h.w = (const __bf16*)lm_head; h.ld_z = p.n_pad; h.ld_w = d->ld_w;
+      h.dzt = (const __bf16*)zt; h.w = (const __bf16*)lm_head; h.ld_z = p.ld_z; h.ld_w = d->ld_w;
       h.n = nc; h.n_pad = n_pad; h.H = H; h.V = V;
       h.splits = p.dh_splits; h.k_per_split = (int)p.dh_k_per_split;
       h.dh = (uint16_t*)d_hidden + c0 * d->ld_hidden; h.ld_dh = d->ld_hidden;
@@ -259,7 +260,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       }
 
       mj::DwArgs w;
-      w.dzt = (const __bf16*)zt; w.hid = hid_c; w.ld_z = p.n_pad; w.ld_hid = d->ld_hidden;
+      w.dzt = (const __bf16*)zt; w.hid = hid_c; w.ld_z = p.ld_z; w.ld_hid = d->ld_hidden;
       w.H = H; w.V = V; w.n = nc;
       w.dw = d_w; w.ld_dw = d->ld_w;
       w.accumulate = (c0 > 0 || (d->flags & MJ_GRPO_FLAG_DW_ACCUMULATE)) ? 1 : 0;
