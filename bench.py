@@ -67,6 +67,11 @@ def main() -> int:
     ap.add_argument("--chunk-tokens", type=int, default=0)
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--skip-masked", action="store_true",
+                    help="time the main loop with MJ_GRPO_FLAG_SKIP_MASKED (tokens without a gradient left out of "
+                         "the backward products); off by default: the headline executes all 6*N*H*V flop")
+    ap.add_argument("--no-skip-masked-extra", action="store_true",
+                    help="do not add the short skip-masked timing to the JSON line")
     ap.add_argument("--no-vendor-gemm", action="store_true",
                     help="skip timing the three bare bf16 products with the vendor GEMM (torch.matmul = hipBLASLt)")
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -101,11 +106,11 @@ def main() -> int:
     n, h, v = cfg.tokens, cfg.hidden, cfg.vocab
     d_w = torch.empty(h, v, dtype=torch.float32, device=dev)
 
-    def step():
+    def step(skip_masked=args.skip_masked):
         return M.grpo_loss_value_and_grad(
             wl["hidden"], wl["lm_head"], wl["target_ids"], wl["old_logps"], wl["advantages"], wl["mask"],
             total_valid_token_count=wl["total_valid_token_count"], seq_shape=wl["seq_shape"],
-            return_token_entropy=cfg.token_entropy, **kw)
+            return_token_entropy=cfg.token_entropy, skip_masked=skip_masked, **kw)
 
     if args.copy_calibration_mib:
         src = torch.empty(args.copy_calibration_mib << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -158,6 +163,23 @@ def main() -> int:
         "roofline": roofline,
         "kernel_ms_per_step": {k: round(v_[0] / args.steps, 3) for k, v_ in prof.items()},
     }
+
+    line["config"]["skip_masked"] = bool(args.skip_masked)
+    if not args.skip_masked and not args.no_skip_masked_extra:
+        # Not the headline: the same step with tokens that cannot carry a gradient (mask 0, advantage 0)
+        # left out of the backward products.  Same outputs; fewer than 6*N*H*V flop executed.
+        for _ in range(2):
+            step(True)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(5):
+            step(True)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t1) / 5 * 1e3
+        live = float(((wl["mask"] != 0) & (wl["advantages"].reshape(wl["mask"].shape) != 0)).float().mean().item())
+        line["skip_masked_extra"] = {"ms_per_step": round(ms, 3), "tokens_per_s": round(n / ms * 1e3, 1),
+                                     "live_token_fraction": round(live, 4),
+                                     "note": "MJ_GRPO_FLAG_SKIP_MASKED; executes 2NHV + 4*live*NHV flop"}
 
     if not args.no_vendor_gemm:
         # Context for the roofline fraction: what the vendor's tuned GEMM reaches on this very

@@ -43,9 +43,16 @@ enum {
 
 enum {
   MJ_GRPO_FLAG_DW_ACCUMULATE = 1u << 0, /* d_lm_head += (grad accumulation, train_step.py:30-33) */
-  MJ_GRPO_FLAG_SFT = 1u << 1            /* masked cross-entropy instead of the clipped surrogate
+  MJ_GRPO_FLAG_SFT = 1u << 1,           /* masked cross-entropy instead of the clipped surrogate
                                            (plugins/sft/jax/sft_module.py:22-45): per-token loss
                                            -logp, advantages/old_logp ignored */
+  MJ_GRPO_FLAG_SKIP_MASKED = 1u << 2    /* tokens whose gradient is zero by construction (mask 0: prompt
+                                           and padding positions, labels of train_modules/__init__.py:120;
+                                           advantage 0 when nothing else feeds the gradient) are moved
+                                           behind the others and left out of the backward products.
+                                           Same outputs (d_lm_head up to summation order); the forward
+                                           still covers every token.  No counterpart in the reference,
+                                           which multiplies the zeros.  Needs a larger workspace. */
 };
 
 typedef struct MjGrpoDesc {

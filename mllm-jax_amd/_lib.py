@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(HERE, "libmj_grpo.so")
 OK = 0
 FLAG_DW_ACCUMULATE = 1 << 0
 FLAG_SFT = 1 << 1
+FLAG_SKIP_MASKED = 1 << 2
 
 EXPORTS = ("mj_grpo_version", "mj_grpo_last_error", "mj_grpo_workspace_bytes", "mj_grpo_forward",
            "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_profile_begin", "mj_grpo_profile_end",

@@ -61,6 +61,9 @@ struct Plan {
   int64_t dh_k_per_split;
   // byte offsets into the workspace
   size_t zy, term, eterm, pm, pl, ps, g, ge, hent, zt, part, total_fwd, total_bwd;
+  // token compaction (MJ_GRPO_FLAG_SKIP_MASKED): slot-order copies of the inputs and outputs
+  bool compact;
+  size_t perm, n_live, hid_p, tgt_p, fin_p[5], fout_p[3], dh_p;
 };
 
 // Splits of the dHidden product over the vocab: its (n/256) x (H/256) tiles rarely fill the 256
@@ -118,7 +121,17 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   p->g = take((size_t)p->n_pad * 4);
   p->ge = take((size_t)p->n_pad * 4);
   p->hent = take((size_t)p->n_pad * 4);
+  p->compact = (d->flags & MJ_GRPO_FLAG_SKIP_MASKED) != 0;
+  if (p->compact) {
+    p->perm = take((size_t)p->N * 4);
+    p->n_live = take(256);
+    p->hid_p = take((size_t)p->N * p->H * 2);
+    p->tgt_p = take((size_t)p->N * 4);
+    for (auto& f : p->fin_p) f = take((size_t)p->N * 4);
+    for (auto& f : p->fout_p) f = take((size_t)p->N * 4);
+  }
   p->total_fwd = o;
+  p->dh_p = take(p->compact ? (size_t)p->N * p->H * 2 : 0);
   p->zt = take((size_t)p->V * p->ld_z * 2);
   p->part = take(p->dh_splits > 1 ? (size_t)p->dh_splits * p->n_pad * p->H * 4 : 0);
   p->total_bwd = o;
@@ -193,17 +206,51 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     if ((rc = enable_lds(mj::k_dw<BM, BN>))) return rc;
   }
 
+  // Token compaction: tokens that cannot carry a gradient go behind the others; everything below
+  // then works on slot-order copies and the backward kernels stop at the device-side count.
+  const int* n_live = nullptr;
+  const int* perm = nullptr;
+  float* out_user[3] = {logp, lse, ent};
+  void* dh_user = d_hidden;
+  int64_t ld_hid = d->ld_hidden, ld_dh = d->ld_hidden;
+  if (p.compact) {
+    perm = (const int*)(ws + p.perm);
+    n_live = (const int*)(ws + p.n_live);
+    mj::CompactArgs c;
+    c.mask = mask; c.adv = (sft || d->entropy_coef != 0.f) ? nullptr : adv; c.n = N;
+    c.perm = (int*)(ws + p.perm); c.n_live = (int*)(ws + p.n_live);
+    mj::k_compact_plan<<<1, 1024, 0, st>>>(c);
+    mj::GatherArgs ga;
+    ga.perm = perm; ga.n = N; ga.H = H; ga.hid = (const uint16_t*)hidden; ga.ld_hid = d->ld_hidden;
+    ga.hid_p = (uint16_t*)(ws + p.hid_p); ga.tgt = targets; ga.tgt_p = (int32_t*)(ws + p.tgt_p);
+    const float* fin[5] = {old_logp, adv, mask, saved_lse, saved_logp};
+    for (int i = 0; i < 5; ++i) { ga.f_in[i] = fin[i]; ga.f_out[i] = (float*)(ws + p.fin_p[i]); }
+    mj::k_gather_tokens<<<N, 256, 0, st>>>(ga);
+    if ((rc = check_launch("token compaction"))) return rc;
+    hidden = ws + p.hid_p; ld_hid = H;
+    targets = (const int32_t*)(ws + p.tgt_p);
+    if (old_logp) old_logp = (const float*)(ws + p.fin_p[0]);
+    if (adv) adv = (const float*)(ws + p.fin_p[1]);
+    mask = (const float*)(ws + p.fin_p[2]);
+    if (saved_lse) saved_lse = (const float*)(ws + p.fin_p[3]);
+    if (saved_logp) saved_logp = (const float*)(ws + p.fin_p[4]);
+    if (logp) logp = (float*)(ws + p.fout_p[0]);
+    if (lse) lse = (float*)(ws + p.fout_p[1]);
+    if (ent) ent = (float*)(ws + p.fout_p[2]);
+    if (bwd) { d_hidden = ws + p.dh_p; ld_dh = H; }
+  }
+
   for (int64_t c0 = 0; c0 < p.N; c0 += p.chunk) {
     const int nc = (int)((p.N - c0 < p.chunk) ? p.N - c0 : p.chunk);
     const int n_pad = (int)rup(nc, 256);
-    const __bf16* hid_c = (const __bf16*)hidden + c0 * d->ld_hidden;
+    const __bf16* hid_c = (const __bf16*)hidden + c0 * ld_hid;
     {
       mj::LogitsArgs a;
-      a.w = (const __bf16*)lm_head; a.hid = hid_c; a.ld_w = d->ld_w; a.ld_hid = d->ld_hidden;
+      a.w = (const __bf16*)lm_head; a.hid = hid_c; a.ld_w = d->ld_w; a.ld_hid = ld_hid;
       a.V = V; a.n = nc; a.H = H; a.cap = d->softcap;
       a.zt = bwd ? zt : nullptr; a.ld_z = p.ld_z;
       a.pm = pm; a.pl = pl; a.ps = ps; a.ld_p = p.n_pad;
-      a.targets = targets + c0; a.zy = zy + c0;
+      a.targets = targets + c0; a.zy = zy + c0; a.n_live = n_live; a.c0 = (int)c0;
       const mj::TileMap map((V + BM - 1) / BM, (nc + BN - 1) / BN, 1);
       Timed t(MJ_GRPO_K_LOGITS_STATS, st);
       mj::k_logits_stats<BM, BN><<<map.items(), mj::kThreads, lds, st>>>(a, map);
@@ -233,10 +280,10 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       z.zt = zt; z.ld_z = p.ld_z;
       z.lse = (mode == kBackwardOnly ? saved_lse : lse) + c0; z.g = g; z.targets = targets + c0;
       z.ge = bonus ? ge : nullptr; z.hent = bonus ? hent : nullptr;
-      z.V = V; z.n = nc; z.n_pad = n_pad; z.cap = d->softcap;
+      z.V = V; z.n = nc; z.n_pad = n_pad; z.cap = d->softcap; z.n_live = n_live; z.c0 = (int)c0;
       {
         Timed t(MJ_GRPO_K_DZ, st);
-        mj::k_dz<<<dim3(n_pad / 256, (V + 63) / 64), 256, 0, st>>>(z);
+        mj::k_dz<<<dim3((V + mj::kDzRows - 1) / mj::kDzRows, n_pad / 256), 256, 0, st>>>(z);
       }
 
       // the split count was planned for a full chunk; a shorter last chunk keeps it (the partial
@@ -245,8 +292,8 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       h.dzt = (const __bf16*)zt; h.w = (const __bf16*)lm_head; h.ld_z = p.ld_z; h.ld_w = d->ld_w;
       h.n = nc; h.n_pad = n_pad; h.H = H; h.V = V;
       h.splits = p.dh_splits; h.k_per_split = (int)p.dh_k_per_split;
-      h.dh = (uint16_t*)d_hidden + c0 * d->ld_hidden; h.ld_dh = d->ld_hidden;
-      h.part = part;
+      h.dh = (uint16_t*)d_hidden + c0 * ld_dh; h.ld_dh = ld_dh;
+      h.part = part; h.n_live = n_live; h.c0 = (int)c0;
       const mj::TileMap mh((nc + BM - 1) / BM, (H + BN - 1) / BN, 0, 2, h.splits);
       {
         Timed t(MJ_GRPO_K_DHIDDEN, st);
@@ -260,9 +307,9 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       }
 
       mj::DwArgs w;
-      w.dzt = (const __bf16*)zt; w.hid = hid_c; w.ld_z = p.ld_z; w.ld_hid = d->ld_hidden;
+      w.dzt = (const __bf16*)zt; w.hid = hid_c; w.ld_z = p.ld_z; w.ld_hid = ld_hid;
       w.H = H; w.V = V; w.n = nc;
-      w.dw = d_w; w.ld_dw = d->ld_w;
+      w.dw = d_w; w.ld_dw = d->ld_w; w.n_live = n_live; w.c0 = (int)c0;
       w.accumulate = (c0 > 0 || (d->flags & MJ_GRPO_FLAG_DW_ACCUMULATE)) ? 1 : 0;
       const mj::TileMap mw((V + BM - 1) / BM, (H + BN - 1) / BN, 0);
       {
@@ -271,6 +318,19 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       }
     }
     if ((rc = check_launch("chunk kernels"))) return rc;
+  }
+  if (p.compact) {
+    mj::ScatterArgs sc;
+    sc.perm = perm; sc.n_live = n_live; sc.n = N; sc.H = H;
+    float* slot[3] = {logp, lse, ent};
+    for (int i = 0; i < 3; ++i) {
+      const bool on = mode != kBackwardOnly && out_user[i] != nullptr;
+      sc.f_in[i] = on ? slot[i] : nullptr;
+      sc.f_out[i] = out_user[i];
+    }
+    sc.dh_p = bwd ? (const uint16_t*)d_hidden : nullptr; sc.dh = (uint16_t*)dh_user; sc.ld_dh = d->ld_hidden;
+    mj::k_scatter_tokens<<<N, 256, 0, st>>>(sc);
+    if ((rc = check_launch("k_scatter_tokens"))) return rc;
   }
   if (mode != kBackwardOnly) {
     {

@@ -61,6 +61,15 @@ MJ_DEV f32x4 load_b128(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
   return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
 
+// Tokens of a chunk that take part in the backward pass, rounded up to whole 256-token tiles:
+// all n_pad of them, or -- when the caller compacted the tokens that carry a gradient to the
+// front -- those up to the device-side count.
+MJ_DEV int live_pad(const int* n_live, int c0, int n_pad) {
+  if (n_live == nullptr) return n_pad;
+  const int left = __builtin_amdgcn_readfirstlane(*n_live) - c0;
+  return min(n_pad, max(left + 255, 0) & ~255);
+}
+
 // ----------------------------------------------------------------------------- logits + stats
 struct LogitsArgs {
   const __bf16* w;       // lm_head [H, ld_w]
@@ -74,6 +83,8 @@ struct LogitsArgs {
   int64_t ld_p;
   const int32_t* targets;   // chunk origin
   float* zy;                // chunk origin: capped logit of the sampled token
+  const int* n_live;        // null, or device count of leading tokens (from token c0 on) that need a backward
+  int c0;
 };
 
 template <int BM, int BN>
@@ -93,6 +104,7 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
   const int vbase = vwave + lhi * 4;             // + mi*32 + (r/4)*8 + r%4
   const bool tail = (m0 + BM > p.V);
   const float inv_cap = p.cap > 0.f ? 1.f / p.cap : 0.f;
+  const int zt_cols = live_pad(p.n_live, p.c0, (p.n + 255) & ~255);
   // this wavefront's 128 rows of logits^T; rows at or past V fall outside and are dropped
   const uint32_t ldz2 = (uint32_t)p.ld_z * 2;
   const int zrows = min(max(p.V - vwave, 0), G::WM);
@@ -160,7 +172,7 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
         if (hit) p.zy[col] = zy;
       }
     }
-    if (p.zt != nullptr) {
+    if (p.zt != nullptr && n0 + wn * G::WN + ni * 32 < zt_cols) {   // tokens past the live ones: dZ is never read
       const uint32_t voff = (uint32_t)((lhi * 4 * p.ld_z + col) * 2);
 #pragma unroll
       for (int mi = 0; mi < G::MI; ++mi)
@@ -308,16 +320,21 @@ struct DzArgs {
   const int32_t* targets;  // chunk origin
   int V, n, n_pad;
   float cap;
+  const int* n_live;   // see live_pad
+  int c0;
 };
 
-// Streaming, in place.  Block = 256 tokens (32 threads x 8) by 64 vocab rows (8 row-lanes x 8
-// steps): every wavefront instruction moves two full 512-byte row segments, and the per-token
-// constants are loaded once per thread.  Tokens at or beyond n (chunk padding) become exact zeros.
+// Streaming, in place.  Block = 256 tokens (32 threads x 8) by kDzRows vocab rows (8 row-lanes x
+// 8 steps per pass): every wavefront instruction moves two full 512-byte row segments, and the
+// per-token constants are loaded once per thread.  Tokens at or beyond n (chunk padding) become
+// exact zeros.  The rows per block are chosen so that the launch is bound by HBM, not by the rate
+// at which workgroups can be dispatched.
+constexpr int kDzRows = 512;
 __global__ __launch_bounds__(256) void k_dz(DzArgs p) {
   const int cx = threadIdx.x & 31, ry = threadIdx.x >> 5;
-  const int t0 = blockIdx.x * 256 + cx * 8;
-  const int v0 = blockIdx.y * 64;
-  if (t0 >= p.n_pad) return;
+  const int t0 = blockIdx.y * 256 + cx * 8;      // vocab blocks vary fastest: whatever part of the
+  const int vblock = blockIdx.x * kDzRows;        // tokens is live, its work spreads over all XCDs
+  if (t0 >= live_pad(p.n_live, p.c0, p.n_pad)) return;
   const float inv_cap2 = p.cap > 0.f ? 1.f / (p.cap * p.cap) : 0.f;
   const bool bonus = p.ge != nullptr;
   float lse[8], g[8], ge[8], hent[8];
@@ -332,6 +349,7 @@ __global__ __launch_bounds__(256) void k_dz(DzArgs p) {
     ge[i] = (bonus && in) ? p.ge[t] : 0.f;
     hent[i] = (bonus && in) ? p.hent[t] : 0.f;
   }
+  for (int v0 = vblock; v0 < min(vblock + kDzRows, p.V); v0 += 64)
 #pragma unroll
   for (int step = 0; step < 8; ++step) {
     const int v = v0 + step * 8 + ry;
@@ -367,14 +385,19 @@ struct DhArgs {
   uint16_t* dh;       // chunk origin [n, ld_dh] bf16 (splits == 1)
   int64_t ld_dh;
   float* part;        // [splits, n_pad, H] fp32 partial sums (splits > 1)
+  const int* n_live;  // see live_pad
+  int c0;
 };
 
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
   using G = GemmTN<BM, BN, kKRow, kRowK>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  // Only token tiles that hold live tokens are walked: the tile list is rebuilt for that many
+  // rows of tiles, so that the live work spreads evenly over the XCDs (ids past its end leave).
+  const TileMap live(live_pad(p.n_live, p.c0, p.n_pad) / BM, map.tiles_n, map.n_first, map.lgm, map.splits);
   int tm, tn, split;
-  if (!map.tile(blockIdx.x, tm, tn, split)) return;
+  if (!live.tile(blockIdx.x, tm, tn, split)) return;
   const int m0 = tm * BM, n0 = tn * BN;
   const int k0 = split * p.k_per_split;
   const int klen = min(p.V - k0, p.k_per_split);
@@ -439,6 +462,8 @@ struct DwArgs {
   float* dw;           // [H, ld_dw] f32
   int64_t ld_dw;
   int accumulate;
+  const int* n_live;   // see live_pad
+  int c0;
 };
 
 // Tile of dW^T: rows = vocab (MFMA row direction), columns = hidden (lanes).  A lane's four
@@ -451,7 +476,8 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
   if (!map.tile(blockIdx.x, tm, tn, split)) return;
   const int m0 = tm * BM, n0 = tn * BN;
   G g;
-  g.run(p.dzt + (int64_t)m0 * p.ld_z, p.V - m0, p.ld_z, p.hid + n0, p.H - n0, p.ld_hid, p.n, smem);
+  const int kn = min(p.n, live_pad(p.n_live, p.c0, (p.n + 255) & ~255));   // tokens past the live ones have dZ = 0
+  g.run(p.dzt + (int64_t)m0 * p.ld_z, p.V - m0, p.ld_z, p.hid + n0, p.H - n0, p.ld_hid, kn, smem);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps descriptors in SGPRs
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
@@ -490,6 +516,83 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
         }
     }
   }
+}
+
+// ----------------------------------------------------------------------------- compaction
+// Optional: tokens whose gradient is zero by construction (mask 0, or advantage 0 where nothing
+// else feeds the gradient) are moved behind the others so that the backward kernels can stop at
+// the count of the rest.  perm[j] = original index of the token in slot j; stable on both sides.
+struct CompactArgs {
+  const float *mask, *adv;   // adv may be null (every unmasked token counts)
+  int n;
+  int* perm;                 // [n]
+  int* n_live;               // [1]
+};
+
+__global__ __launch_bounds__(1024) void k_compact_plan(CompactArgs p) {
+  __shared__ int cnt[1024];
+  const int t = threadIdx.x;
+  const int seg = (p.n + 1023) / 1024;
+  const int b = min(t * seg, p.n), e = min(b + seg, p.n);
+  int c = 0;
+  for (int i = b; i < e; ++i) c += (p.mask[i] != 0.f && (p.adv == nullptr || p.adv[i] != 0.f)) ? 1 : 0;
+  cnt[t] = c;
+  __syncthreads();
+  for (int o = 1; o < 1024; o <<= 1) {          // inclusive scan
+    const int v = t >= o ? cnt[t - o] : 0;
+    __syncthreads();
+    cnt[t] += v;
+    __syncthreads();
+  }
+  const int total = cnt[1023];
+  int live = cnt[t] - c;                        // live tokens before this segment
+  int dead = total + (b - live);                // slot of this segment's first dead token
+  for (int i = b; i < e; ++i) {
+    const bool ok = p.mask[i] != 0.f && (p.adv == nullptr || p.adv[i] != 0.f);
+    if (ok) p.perm[live++] = i; else p.perm[dead++] = i;
+  }
+  if (t == 0) p.n_live[0] = total;
+}
+
+struct GatherArgs {
+  const int* perm;
+  int n, H;
+  const uint16_t* hid; int64_t ld_hid;     // [n, ld_hid] -> hid_p [n, H]
+  uint16_t* hid_p;
+  const int32_t* tgt; int32_t* tgt_p;
+  const float *f_in[5];                    // old_logp, adv, mask, saved_lse, saved_logp (any may be null)
+  float* f_out[5];
+};
+
+// one workgroup per slot: copies the token's hidden row (16 bytes per thread and step) and scalars
+__global__ __launch_bounds__(256) void k_gather_tokens(GatherArgs p) {
+  const int j = blockIdx.x, src = p.perm[j];
+  const u32x4* in = (const u32x4*)(p.hid + (int64_t)src * p.ld_hid);
+  u32x4* out = (u32x4*)(p.hid_p + (int64_t)j * p.H);
+  for (int c = threadIdx.x; c < (p.H >> 3); c += 256) out[c] = in[c];
+  if (threadIdx.x == 0) p.tgt_p[j] = p.tgt[src];
+  if (threadIdx.x < 5 && p.f_in[threadIdx.x] != nullptr) p.f_out[threadIdx.x][j] = p.f_in[threadIdx.x][src];
+}
+
+struct ScatterArgs {
+  const int* perm;
+  const int* n_live;
+  int n, H;
+  const float* f_in[3];                    // logp, lse, entropy in slot order (any may be null)
+  float* f_out[3];
+  const uint16_t* dh_p;                    // [n, H] slot order, or null (no backward)
+  uint16_t* dh; int64_t ld_dh;
+};
+
+// inverse of the gather for the outputs; tokens behind the live ones get a zero d_hidden row
+__global__ __launch_bounds__(256) void k_scatter_tokens(ScatterArgs p) {
+  const int j = blockIdx.x, dst = p.perm[j];
+  if (threadIdx.x < 3 && p.f_in[threadIdx.x] != nullptr) p.f_out[threadIdx.x][dst] = p.f_in[threadIdx.x][j];
+  if (p.dh_p == nullptr) return;
+  const bool live = j < *p.n_live;
+  const u32x4* in = (const u32x4*)(p.dh_p + (int64_t)j * p.H);
+  u32x4* out = (u32x4*)(p.dh + (int64_t)dst * p.ld_dh);
+  for (int c = threadIdx.x; c < (p.H >> 3); c += 256) out[c] = live ? in[c] : u32x4{0u, 0u, 0u, 0u};
 }
 
 // ----------------------------------------------------------------------------- sampling

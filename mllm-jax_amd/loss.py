@@ -57,7 +57,7 @@ class _Prepared:
     def __init__(self, hidden, lm_head, target_ids, old_logps, advantages, mask, *,
                  total_valid_token_count, epsilon_low, epsilon_high, temperature,
                  final_logit_softcap, seq_shape, chunk_tokens, sft=False, accumulate=False,
-                 entropy_coef=0.0, entropy_token_count=None):
+                 entropy_coef=0.0, entropy_token_count=None, skip_masked=False):
         if hidden.device.type != "cuda":
             raise RuntimeError("grpo_fused_loss needs tensors on an MI355X device (got "
                                f"{hidden.device}); there is no CPU path")
@@ -116,7 +116,8 @@ class _Prepared:
         if entropy_coef != 0.0 or entropy_token_count is not None:
             cnt = float(self.mask.sum().item()) if entropy_token_count is None else float(entropy_token_count)
             d.inv_entropy_count = 1.0 / (cnt + 1e-8)             # ppo/module.py:77
-        d.flags = (_lib.FLAG_SFT if sft else 0) | (_lib.FLAG_DW_ACCUMULATE if accumulate else 0)
+        d.flags = (_lib.FLAG_SFT if sft else 0) | (_lib.FLAG_DW_ACCUMULATE if accumulate else 0) \
+            | (_lib.FLAG_SKIP_MASKED if skip_masked else 0)
         self.desc = d
         self.logp = torch.empty(n, dtype=torch.float32, device=dev)
         self.lse = torch.empty(n, dtype=torch.float32, device=dev)
@@ -174,7 +175,7 @@ class _Prepared:
 
 _DEFAULTS = dict(total_valid_token_count=None, epsilon_low=0.2, epsilon_high=0.3, temperature=1.0,
                  final_logit_softcap=None, seq_shape=None, chunk_tokens=None, entropy_coef=0.0,
-                 entropy_token_count=None)
+                 entropy_token_count=None, skip_masked=False)
 
 
 def grpo_loss_value_and_grad(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
@@ -188,7 +189,9 @@ def grpo_loss_value_and_grad(hidden, lm_head, target_ids, old_logps, advantages,
     One fused pass: 6*N*H*V flop, 16-bit logits of at most `chunk_tokens` tokens in the workspace.
     `entropy_coef` != 0 subtracts entropy_coef * sum(H_t*mask)/(sum(mask)+1e-8) from the loss
     (the entropy bonus of plugins/training/ppo/module.py:75-77, :140), gradient included; that
-    entropy is returned as metrics["masked_mean_entropy"]."""
+    entropy is returned as metrics["masked_mean_entropy"].
+    `skip_masked=True` leaves tokens that cannot carry a gradient (mask 0; advantage 0) out of the
+    backward products: same results, less work when the batch holds prompt / padding positions."""
     opts = {**_DEFAULTS, **kw}
     p = _Prepared(hidden, lm_head, target_ids, old_logps, advantages, mask,
                   accumulate=accumulate_into is not None, **opts)
@@ -311,13 +314,14 @@ class TrainGRPOModule:
                  ref_model: Any = None, beta: float = 0.04, temperature: float = 1.0,
                  max_lengths: float = 2048, epsilon_low: float = 0.2, epsilon_high: float = 0.3,
                  entropy_threshold: float = 0.3, final_logit_softcap: Optional[float] = None,
-                 chunk_tokens: Optional[int] = None):
+                 chunk_tokens: Optional[int] = None, skip_masked: bool = False):
         self.model, self.lm_head = model, lm_head
         self.pad_token_id, self.num_pre_Q, self.ref_model, self.beta = pad_token_id, num_pre_Q, ref_model, beta
         self.temperature, self.max_lengths = temperature, max_lengths
         self.epsilon_low, self.epsilon_high = epsilon_low, epsilon_high
         self.entropy_threshold = entropy_threshold
         self.final_logit_softcap, self.chunk_tokens = final_logit_softcap, chunk_tokens
+        self.skip_masked = skip_masked
 
     def __call__(self, inputs: Mapping[str, Any]) -> dict:
         input_ids, labels = inputs["input_ids"], inputs["labels"]
@@ -333,7 +337,7 @@ class TrainGRPOModule:
             total_valid_token_count=inputs.get("total_valid_token_count"),
             epsilon_low=self.epsilon_low, epsilon_high=self.epsilon_high, temperature=self.temperature,
             final_logit_softcap=self.final_logit_softcap, seq_shape=(b, l - 1),
-            chunk_tokens=self.chunk_tokens)
+            chunk_tokens=self.chunk_tokens, skip_masked=self.skip_masked)
 
 
 class PPOActorCriticModule:
@@ -350,7 +354,9 @@ class PPOActorCriticModule:
     def __init__(self, model: Callable, lm_head, value_head, temperature: float = 1.0,
                  epsilon_low: float = 0.2, epsilon_high: float = 0.2, value_coef: float = 0.5,
                  value_clip_range: Optional[float] = 0.2, entropy_coef: float = 0.0,
-                 final_logit_softcap: Optional[float] = None, chunk_tokens: Optional[int] = None):
+                 final_logit_softcap: Optional[float] = None, chunk_tokens: Optional[int] = None,
+                 skip_masked: bool = False):
+        self.skip_masked = skip_masked
         self.model, self.lm_head, self.value_head = model, lm_head, value_head
         self.temperature, self.epsilon_low, self.epsilon_high = temperature, epsilon_low, epsilon_high
         self.value_coef, self.value_clip_range, self.entropy_coef = value_coef, value_clip_range, entropy_coef
@@ -395,7 +401,8 @@ class PPOActorCriticModule:
                       total_valid_token_count=float(tv) if tv is not None else float(msum.item()),
                       epsilon_low=self.epsilon_low, epsilon_high=self.epsilon_high,
                       temperature=self.temperature, final_logit_softcap=self.final_logit_softcap,
-                      seq_shape=(b, t), chunk_tokens=self.chunk_tokens, entropy_coef=self.entropy_coef,
+                      seq_shape=(b, t), chunk_tokens=self.chunk_tokens, skip_masked=self.skip_masked,
+                      entropy_coef=self.entropy_coef,
                       entropy_token_count=float(msum.item()) if self.entropy_coef != 0.0 or tv is None else None)
         want = torch.is_grad_enabled() and (hidden.requires_grad or w.requires_grad)
         fused = _FusedLossFn.apply(hidden[:, :-1, :].reshape(b * t, -1), w, p, want)   # policy - coef * entropy
