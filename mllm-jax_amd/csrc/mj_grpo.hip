@@ -97,6 +97,8 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
     return fail(MJ_GRPO_ERR_UNSUPPORTED, "temperature %g unsupported (only 1.0)", (double)d->temperature);
   if (d->softcap < 0.f || !isfinite(d->softcap)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "softcap must be >= 0");
   if (d->chunk_tokens < 0) return fail(MJ_GRPO_ERR_SHAPE, "chunk_tokens must be >= 0");
+  if (d->flags & ~(uint32_t)(MJ_GRPO_FLAG_DW_ACCUMULATE | MJ_GRPO_FLAG_SFT | MJ_GRPO_FLAG_SKIP_MASKED))
+    return fail(MJ_GRPO_ERR_UNSUPPORTED, "unknown bits in flags (0x%x)", d->flags);
   if (!isfinite(d->inv_total_valid_tokens)) return fail(MJ_GRPO_ERR_SHAPE, "inv_total_valid_tokens not finite");
   if (!isfinite(d->entropy_coef) || !isfinite(d->inv_entropy_count) || d->inv_entropy_count < 0.f)
     return fail(MJ_GRPO_ERR_SHAPE, "entropy_coef / inv_entropy_count not finite");

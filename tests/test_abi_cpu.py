@@ -59,7 +59,8 @@ def test_workspace_sizes_scale_with_chunk(lib):
     (dict(vocab=508, ld_w=508), 3), (dict(hidden=60, ld_hidden=60), 3), (dict(ld_hidden=68), 3),
     (dict(temperature=0.7), 5), (dict(softcap=-1.0), 5), (dict(chunk_tokens=-5), 2),
     (dict(inv_total_valid_tokens=float("inf")), 2),
-    (dict(entropy_coef=float("nan")), 2), (dict(inv_entropy_count=-1.0), 2),
+    (dict(entropy_coef=float("nan")), 2), (dict(inv_entropy_count=-1.0), 2), (dict(flags=1 << 7), 5),
+    (dict(vocab=1 << 22, ld_w=1 << 22), 2), (dict(chunk_tokens=1 << 21), 2),
 ])
 def test_bad_descriptors(lib, kw, code):
     with pytest.raises(lib.MjGrpoError) as e:
@@ -139,3 +140,13 @@ def test_sampler_argument_checks_before_any_launch(lib):
     assert h.mj_sample_top_k(fake, 512, 4, 40, 50, 1.0, None, fake, None, None, None) == 5      # k > vocab
     assert h.mj_sample_top_k(fake, 512, 4, 512, 50, 0.0, None, fake, None, None, None) == 5
     assert h.mj_sample_top_k(fake, 512, 4, 512, 50, 1.0, None, None, None, None, None) == 1
+
+
+def test_skip_masked_flag_enlarges_the_workspace(lib):
+    d = _desc(lib)
+    fwd0, both0 = lib.workspace_bytes(d)
+    d.flags = lib.FLAG_SKIP_MASKED
+    fwd1, both1 = lib.workspace_bytes(d)
+    n, h = d.n_tokens, d.hidden
+    assert fwd1 >= fwd0 + n * h * 2 + n * 4 * 10          # slot-order hidden copy, permutation, per-token copies
+    assert both1 - fwd1 >= both0 - fwd0 + n * h * 2       # slot-order d_hidden
