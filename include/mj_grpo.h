@@ -19,7 +19,7 @@
  * old_logp[N] f32 or NULL (NULL = on-policy, ratio == 1, train_modules/__init__.py:161-165),
  * advantages[N] f32 (the reference's [B] broadcast per token, :173), mask[N] f32 in {0,1}.
  * Requirements: H % 8 == 0, V % 8 == 0, ld_hidden % 8 == 0, ld_w % 8 == 0,
- * bf16 pointers, d_lm_head and the workspace 16-byte aligned, temperature == 1.
+ * bf16 pointers, d_lm_head and the workspace 16-byte aligned, temperature > 0.
  */
 #ifndef MJ_GRPO_H
 #define MJ_GRPO_H
@@ -37,7 +37,7 @@ enum {
   MJ_GRPO_ERR_SHAPE = 2,       /* N/H/V/ld out of range */
   MJ_GRPO_ERR_ALIGN = 3,       /* pointer or leading dimension not 16-byte aligned */
   MJ_GRPO_ERR_WORKSPACE = 4,   /* workspace missing or too small */
-  MJ_GRPO_ERR_UNSUPPORTED = 5, /* e.g. temperature != 1 */
+  MJ_GRPO_ERR_UNSUPPORTED = 5, /* e.g. temperature <= 0, unknown flag, entropy bonus with temperature != 1 */
   MJ_GRPO_ERR_HIP = 6          /* a HIP call or kernel launch failed */
 };
 
@@ -64,7 +64,8 @@ typedef struct MjGrpoDesc {
   int64_t chunk_tokens;  /* tokens whose 16-bit logits live in the workspace at once; 0 = default */
   float eps_low;         /* TrainGRPOModule.epsilon_low  (train_modules/__init__.py:92) */
   float eps_high;        /* TrainGRPOModule.epsilon_high (:93) */
-  float temperature;     /* must be 1 (:91) */
+  float temperature;     /* T > 0 (:91).  As in the reference, logp = log_softmax(z)[y] / T (:124-126) while the
+                            entropy is that of softmax(z / T) (:136); lse[] is always logsumexp(z) */
   float softcap;         /* final-logit softcap, 0 = off (gemma/transformer.py:337-339) */
   float inv_total_valid_tokens; /* 1 / total_valid_token_count (:179-180) */
   float grad_loss_scale; /* upstream d(loss); 1 for a terminal loss */

@@ -60,7 +60,7 @@ struct Plan {
   int dh_splits;          // vocab splits of the dHidden product (1 = none)
   int64_t dh_k_per_split;
   // byte offsets into the workspace
-  size_t zy, term, eterm, pm, pl, ps, g, ge, hent, zt, part, total_fwd, total_bwd;
+  size_t zy, term, eterm, pm, pl, ps, plt, g, ge, hent, zt, part, total_fwd, total_bwd;
   // token compaction (MJ_GRPO_FLAG_SKIP_MASKED): slot-order copies of the inputs and outputs
   bool compact;
   size_t perm, n_live, hid_p, tgt_p, fin_p[5], fout_p[3], dh_p;
@@ -93,8 +93,10 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
     return fail(MJ_GRPO_ERR_SHAPE, "leading dimension smaller than row length");
   if (d->hidden % 8 || d->vocab % 8 || d->ld_hidden % 8 || d->ld_w % 8)
     return fail(MJ_GRPO_ERR_ALIGN, "hidden, vocab, ld_hidden and ld_w must be multiples of 8");
-  if (d->temperature != 1.0f)
-    return fail(MJ_GRPO_ERR_UNSUPPORTED, "temperature %g unsupported (only 1.0)", (double)d->temperature);
+  if (!(d->temperature > 0.f) || !isfinite(d->temperature))
+    return fail(MJ_GRPO_ERR_UNSUPPORTED, "temperature must be positive and finite (got %g)", (double)d->temperature);
+  if (d->temperature != 1.0f && d->entropy_coef != 0.f)
+    return fail(MJ_GRPO_ERR_UNSUPPORTED, "an entropy bonus needs temperature 1 (got %g)", (double)d->temperature);
   if (d->softcap < 0.f || !isfinite(d->softcap)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "softcap must be >= 0");
   if (d->chunk_tokens < 0) return fail(MJ_GRPO_ERR_SHAPE, "chunk_tokens must be >= 0");
   if (d->flags & ~(uint32_t)(MJ_GRPO_FLAG_DW_ACCUMULATE | MJ_GRPO_FLAG_SFT | MJ_GRPO_FLAG_SKIP_MASKED))
@@ -120,6 +122,7 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   p->pm = take((size_t)p->parts * p->n_pad * 4);
   p->pl = take((size_t)p->parts * p->n_pad * 4);
   p->ps = take((size_t)p->parts * p->n_pad * 4);
+  p->plt = take(d->temperature != 1.0f ? (size_t)p->parts * p->n_pad * 4 : 0);
   p->g = take((size_t)p->n_pad * 4);
   p->ge = take((size_t)p->n_pad * 4);
   p->hent = take((size_t)p->n_pad * 4);
@@ -196,6 +199,8 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
   float* pm = (float*)(ws + p.pm);
   float* pl = (float*)(ws + p.pl);
   float* ps = (float*)(ws + p.ps);
+  float* plt = (float*)(ws + p.plt);
+  const float inv_t = d->temperature == 1.0f ? 1.0f : 1.0f / d->temperature;
   float* g = (float*)(ws + p.g);
   uint16_t* zt = (uint16_t*)(ws + p.zt);
   float* part = (float*)(ws + p.part);
@@ -251,7 +256,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       a.w = (const __bf16*)lm_head; a.hid = hid_c; a.ld_w = d->ld_w; a.ld_hid = ld_hid;
       a.V = V; a.n = nc; a.H = H; a.cap = d->softcap;
       a.zt = bwd ? zt : nullptr; a.ld_z = p.ld_z;
-      a.pm = pm; a.pl = pl; a.ps = ps; a.ld_p = p.n_pad;
+      a.pm = pm; a.pl = pl; a.ps = ps; a.plt = plt; a.inv_t = inv_t; a.ld_p = p.n_pad;
       a.targets = targets + c0; a.zy = zy + c0; a.n_live = n_live; a.c0 = (int)c0;
       const mj::TileMap map((V + BM - 1) / BM, (nc + BN - 1) / BN, 1);
       Timed t(MJ_GRPO_K_LOGITS_STATS, st);
@@ -259,7 +264,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     }
     if (mode != kBackwardOnly) {
       mj::FinalizeArgs f;
-      f.pm = pm; f.pl = pl; f.ps = ps; f.ld_p = p.n_pad; f.parts = (int)p.parts;
+      f.pm = pm; f.pl = pl; f.ps = ps; f.plt = plt; f.inv_t = inv_t; f.ld_p = p.n_pad; f.parts = (int)p.parts;
       f.n = nc; f.n_pad = n_pad; f.zy = zy + c0;
       f.old_logp = old_logp ? old_logp + c0 : nullptr;
       f.adv = adv ? adv + c0 : nullptr; f.mask = mask + c0;
@@ -275,7 +280,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       Timed t(MJ_GRPO_K_FINALIZE, st);
       mj::k_coeff_from_saved<<<(n_pad + 255) / 256, 256, 0, st>>>(
           saved_logp + c0, old_logp ? old_logp + c0 : nullptr, adv ? adv + c0 : nullptr, mask + c0, nc, n_pad,
-          d->eps_low, d->eps_high, d->inv_total_valid_tokens, gscale, sft ? 1 : 0, g);
+          d->eps_low, d->eps_high, d->inv_total_valid_tokens, gscale * inv_t, sft ? 1 : 0, g);
     }
     if (bwd) {
       mj::DzArgs z;

@@ -80,6 +80,8 @@ struct LogitsArgs {
   uint16_t* zt;          // [V, ld_z] half logits^T of the chunk, or nullptr (forward only)
   int64_t ld_z;
   float *pm, *pl, *ps;   // per (vocab half-tile, token) partial max / sum e / sum e*z, ld = ld_p
+  float* plt;            // temperature != 1 only: sum e^((z-max)/T), and ps then holds sum e^((z-max)/T)*z
+  float inv_t;           // 1 / temperature
   int64_t ld_p;
   const int32_t* targets;   // chunk origin
   float* zy;                // chunk origin: capped logit of the sampled token
@@ -149,11 +151,31 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
       }
     l += __shfl_xor(l, 32);
     s += __shfl_xor(s, 32);
+    float lt = 0.f;
+    if (p.inv_t != 1.f) {
+      // The reference takes the log-prob from softmax(z) but the entropy from softmax(z / T)
+      // (train_modules/__init__.py:124-126, :136): a second pair of sums, only when T != 1.
+      asm volatile("");
+      const float kt = kLog2e * p.inv_t, mxt = mx * kt;
+      s = 0.f;
+#pragma unroll
+      for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float z = g.acc[mi][ni][r];
+          const float e = __builtin_amdgcn_exp2f(fmaf(z, kt, -mxt));
+          lt += e;
+          s = fmaf(e, z, s);
+        }
+      lt += __shfl_xor(lt, 32);
+      s += __shfl_xor(s, 32);
+    }
     if (lhi == 0) {
       const int64_t o = (int64_t)(tm * 2 + wm) * p.ld_p + col;
       p.pm[o] = mx;
       p.pl[o] = l;
       p.ps[o] = s;
+      if (p.inv_t != 1.f) p.plt[o] = lt;
     }
     // The sampled token's logit: exactly one lane of one tile holds it.  Few wavefronts have a
     // hit at all (32 tokens x 128 rows out of V), so the register search sits behind a vote.
@@ -186,6 +208,8 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
 // ----------------------------------------------------------------------------- finalize
 struct FinalizeArgs {
   const float *pm, *pl, *ps;   // [parts, ld_p]
+  const float* plt;            // [parts, ld_p], temperature != 1 only
+  float inv_t;
   int64_t ld_p;
   int parts, n, n_pad;         // tokens in chunk, padded count (g is written for all n_pad)
   const float* zy;             // [n] chunk-local
@@ -202,10 +226,11 @@ struct FinalizeArgs {
 
 // block = (64 tokens) x (4 slices of the partial list)
 __global__ __launch_bounds__(256) void k_finalize(FinalizeArgs p) {
-  __shared__ float sm[4][64], sl[4][64], ss[4][64];
+  __shared__ float sm[4][64], sl[4][64], ss[4][64], st[4][64];
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int t = blockIdx.x * 64 + tx;
-  float m = kNegBig, l = 0.f, s = 0.f;
+  const bool tempered = p.inv_t != 1.f;   // then s and lt are sums under softmax(z / T)
+  float m = kNegBig, l = 0.f, s = 0.f, lt = 0.f;
   if (t < p.n) {
     for (int q = ty; q < p.parts; q += 4) {
       const int64_t o = (int64_t)q * p.ld_p + t;
@@ -213,11 +238,17 @@ __global__ __launch_bounds__(256) void k_finalize(FinalizeArgs p) {
       const float mn = fmaxf(m, mq);
       const float a = __expf(m - mn), b = __expf(mq - mn);
       l = l * a + lq * b;
-      s = s * a + sq * b;
+      if (tempered) {
+        const float at = __expf((m - mn) * p.inv_t), bt = __expf((mq - mn) * p.inv_t);
+        lt = lt * at + p.plt[o] * bt;
+        s = s * at + sq * bt;
+      } else {
+        s = s * a + sq * b;
+      }
       m = mn;
     }
   }
-  sm[ty][tx] = m; sl[ty][tx] = l; ss[ty][tx] = s;
+  sm[ty][tx] = m; sl[ty][tx] = l; ss[ty][tx] = s; st[ty][tx] = lt;
   __syncthreads();
   if (ty != 0) return;
   if (t >= p.n) {
@@ -226,18 +257,21 @@ __global__ __launch_bounds__(256) void k_finalize(FinalizeArgs p) {
     return;
   }
   float M = fmaxf(fmaxf(sm[0][tx], sm[1][tx]), fmaxf(sm[2][tx], sm[3][tx]));
-  float L = 0.f, S = 0.f;
+  float L = 0.f, S = 0.f, LT = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const float w = __expf(sm[i][tx] - M);
+    const float wt = tempered ? __expf((sm[i][tx] - M) * p.inv_t) : w;
     L += sl[i][tx] * w;
-    S += ss[i][tx] * w;
+    S += ss[i][tx] * wt;
+    LT += st[i][tx] * wt;
   }
   const float lse = M + __logf(L);
-  const float logp = p.zy[t] - lse;
+  const float logp = (p.zy[t] - lse) * p.inv_t;     // division after the log-softmax (:124-126)
   p.lse[t] = lse;
   p.logp[t] = logp;
-  const float H = lse - S / L;                    // = -sum p log p  (reference adds 1e-9 inside the log)
+  // entropy of softmax(z / T): log sum e^(z/T) - sum p z / T  (reference adds 1e-9 inside the log)
+  const float H = tempered ? (M * p.inv_t + __logf(LT)) - (S / LT) * p.inv_t : lse - S / L;
   if (p.ent != nullptr) p.ent[t] = H;
   const float mk = p.mask[t];
   p.eterm[t] = H * mk * p.inv_ent_cnt;
@@ -259,7 +293,7 @@ __global__ __launch_bounds__(256) void k_finalize(FinalizeArgs p) {
     g = active ? -mk * p.inv_tv * adv * ratio : 0.f;
   }
   p.term[t] = term;
-  if (p.g != nullptr) p.g[t] = g * p.gscale;
+  if (p.g != nullptr) p.g[t] = g * p.gscale * p.inv_t;   // dlogp/dz = (onehot - softmax(z)) / T
 }
 
 // dloss/dlogp from a saved forward (separate backward entry point)
@@ -267,6 +301,7 @@ __global__ __launch_bounds__(256) void k_coeff_from_saved(const float* logp, con
                                                           const float* adv, const float* mask, int n,
                                                           int n_pad, float eps_low, float eps_high,
                                                           float inv_tv, float gscale, int sft, float* g) {
+  // gscale carries 1 / temperature as well (see k_finalize)
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= n_pad) return;
   float out = 0.f;

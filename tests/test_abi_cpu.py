@@ -57,7 +57,7 @@ def test_workspace_sizes_scale_with_chunk(lib):
 @pytest.mark.parametrize("kw,code", [
     (dict(n_tokens=0), 2), (dict(vocab=-8), 2), (dict(ld_w=256), 2),
     (dict(vocab=508, ld_w=508), 3), (dict(hidden=60, ld_hidden=60), 3), (dict(ld_hidden=68), 3),
-    (dict(temperature=0.7), 5), (dict(softcap=-1.0), 5), (dict(chunk_tokens=-5), 2),
+    (dict(temperature=0.0), 5), (dict(temperature=0.7, entropy_coef=0.1, inv_entropy_count=0.1), 5), (dict(softcap=-1.0), 5), (dict(chunk_tokens=-5), 2),
     (dict(inv_total_valid_tokens=float("inf")), 2),
     (dict(entropy_coef=float("nan")), 2), (dict(inv_entropy_count=-1.0), 2), (dict(flags=1 << 7), 5),
     (dict(vocab=1 << 22, ld_w=1 << 22), 2), (dict(chunk_tokens=1 << 21), 2),

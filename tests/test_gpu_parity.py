@@ -255,7 +255,7 @@ def test_error_paths_on_device():
     d = _dev()
     hid, w, y, adv, mask = _case(20, 16, 8, 296, 2)
     with pytest.raises(MjGrpoError):
-        M.grpo_fused_loss(hid.to(d), w.to(d), y.to(d), None, adv.to(d), mask.to(d), temperature=0.5)
+        M.grpo_fused_loss(hid.to(d), w.to(d), y.to(d), None, adv.to(d), mask.to(d), temperature=0.0)
     with pytest.raises(MjGrpoError):    # vocab not a multiple of 8
         M.grpo_fused_loss(hid.to(d), w[:, :291].contiguous().to(d), y.to(d) % 291, None, adv.to(d), mask.to(d))
     with pytest.raises(RuntimeError):   # CPU tensors: no fallback
@@ -283,3 +283,15 @@ def test_group_advantages_on_device():
     assert out[0].item() == 0.0 and out.dtype == torch.float32
     with pytest.raises(ValueError):
         M.compute_grpo_advantages_by_group_id(rewards=torch.zeros(4, device=d), group_ids=torch.zeros(3))
+
+
+@pytest.mark.parametrize("temp", [0.7, 2.0])
+def test_temperature_divides_logp_and_tempers_the_entropy(temp):
+    # logp = log_softmax(z)[y] / T, entropy of softmax(z / T) (train_modules/__init__.py:124-126, :136)
+    hid, w, y, adv, mask = _case(31, 520, 72, 1544, 4)
+    old = torch.from_numpy(_ref_logp(hid, w, y, temperature=temp)).float() + 0.1 * torch.randn(520, generator=torch.Generator().manual_seed(3))
+    met, dh, dw, ref = _check(hid, w, y, old, adv, mask, seq_shape=(4, 130), chunk_tokens=256, temperature=temp,
+                              epsilon_low=0.2, epsilon_high=0.3)
+    plain = O.grpo_loss(hid.float().numpy(), w.float().numpy(), y.numpy(), None, np.zeros(520), np.ones(520), with_grads=False)
+    np.testing.assert_allclose(met["per_token_logps"].reshape(-1), plain["per_token_logps"] / temp, atol=1e-3)
+    assert np.abs(met["token_entropy"].reshape(-1) - plain["token_entropy"]).max() > 0.05      # it is a different entropy
