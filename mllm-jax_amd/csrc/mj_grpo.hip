@@ -67,11 +67,11 @@ struct Plan {
 };
 
 // Splits of the dHidden product over the vocab: its (n/256) x (H/256) tiles rarely fill the 256
-// CUs in whole rounds, so K = V is cut into the fewest pieces (<= 8) that waste < 4% of a round.
+// CUs in whole rounds, so K = V is cut into the fewest pieces (<= 32) that waste < 4% of a round.
 int pick_splits(int64_t tiles) {
   int best = 1;
   double best_eff = 0.0;
-  for (int s = 1; s <= 8; ++s) {
+  for (int s = 1; s <= 32; ++s) {
     const int64_t items = tiles * s, rounds = (items + 255) / 256;
     const double eff = (double)items / (double)(rounds * 256);
     if (eff > best_eff + 1e-9) { best_eff = eff; best = s; }
