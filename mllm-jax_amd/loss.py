@@ -308,7 +308,11 @@ class TrainGRPOModule:
     Qwen2Model returns before lm_head, qwen2/modular_qwen2.py:161) and `lm_head` is the
     [H,V] kernel (or a zero-argument callable returning it).  `__call__(inputs)` takes the
     reference's batch dict (input_ids, attention_mask, labels, advantages and optionally
-    old_per_token_logps, total_valid_token_count) and returns its metrics dict."""
+    old_per_token_logps, total_valid_token_count) and returns its metrics dict.
+
+    `ref_model` and `beta` are accepted and, as in the reference, have no effect on the loss: the
+    reference evaluates the reference model's log-probs (:129-132) but no KL term enters `loss`
+    (:176-180).  `pad_token_id`, `num_pre_Q`, `max_lengths`, `entropy_threshold` are unused there too."""
 
     def __init__(self, model: Callable, lm_head, pad_token_id: float = 0, num_pre_Q: int = 1,
                  ref_model: Any = None, beta: float = 0.04, temperature: float = 1.0,
