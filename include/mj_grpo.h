@@ -121,13 +121,30 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
                      const float* mask, const float* lse, const float* logp, void* d_hidden,
                      float* d_lm_head, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Group-normalised advantages on the device: advantages[i] = (r_i - mean_g) / (std_g + eps) over
- * the samples that share group_ids[i] (population std; any int ids, any group sizes).  Replaces
- * compute_grpo_advantages_by_group_id (plugins/training/advantage/grpo.py:8-52), which the
- * runner evaluates in host NumPy (runner/grpo_gsm8k.py:680).  rewards, advantages: float32 [b];
- * group_ids: int32 [b]. */
+/* Sequence-level advantage estimators on the device (host NumPy in the reference, evaluated by the
+ * runner at runner/grpo_gsm8k.py:680).  rewards, advantages: float32 [b]; group_ids: int32 [b] (any
+ * ids, any group sizes; unused by MJ_GRPO_ADV_GLOBAL).  b <= 65536.
+ *   MJ_GRPO_ADV_GRPO    (r - mean_g) / (std_g + eps), population std     advantage/grpo.py:8-52
+ *   MJ_GRPO_ADV_GLOBAL  (r - mean) / (std + eps)                          advantage/estimators.py:37-55
+ *   MJ_GRPO_ADV_RLOO    r - mean of the others in the group (group mean for singletons); whiten != 0
+ *                       then centres and scales over the batch            estimators.py:58-103, :137-157
+ *   MJ_GRPO_ADV_DAPO    GRPO + alpha * GLOBAL                             estimators.py:106-134
+ * clip_range > 0 clips the result to [-clip_range, clip_range] (estimators.py:28-34). */
+enum { MJ_GRPO_ADV_GRPO = 0, MJ_GRPO_ADV_GLOBAL = 1, MJ_GRPO_ADV_RLOO = 2, MJ_GRPO_ADV_DAPO = 3 };
+int mj_grpo_advantages(int mode, const float* rewards, const int32_t* group_ids, float* advantages,
+                       int64_t b, float eps, float alpha, int whiten, float clip_range, void* stream);
+
+/* mj_grpo_advantages(MJ_GRPO_ADV_GRPO, ...): compute_grpo_advantages_by_group_id. */
 int mj_grpo_group_advantages(const float* rewards, const int32_t* group_ids, float* advantages,
                              int64_t b, float eps, void* stream);
+
+/* Token-level GAE (compute_gae_advantages, advantage/estimators.py:180-240; the sequence reward is
+ * placed on the last completion token, build_token_rewards_from_final, :160-177).  rewards [b];
+ * values, completion_mask, advantages, returns: float32 [b, t] row-major.  normalize != 0 centres and
+ * scales the advantages over the completion tokens and zeroes the others; clip_range > 0 clips. */
+int mj_grpo_gae(const float* rewards, const float* values, const float* completion_mask,
+                float* advantages, float* returns, int64_t b, int64_t t, float gamma, float gae_lambda,
+                int normalize, float eps, float clip_range, void* stream);
 
 /* Optional per-kernel timing (bench and profiling; no counterpart in the reference, whose only
  * timers are wall-clock phase timers, plugins/training/runner/grpo_gsm8k.py:615-792).

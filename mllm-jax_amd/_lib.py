@@ -17,7 +17,7 @@ FLAG_SKIP_MASKED = 1 << 2
 
 EXPORTS = ("mj_grpo_version", "mj_grpo_last_error", "mj_grpo_workspace_bytes", "mj_grpo_forward",
            "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_profile_begin", "mj_grpo_profile_end",
-           "mj_grpo_group_advantages", "mj_rmsnorm_forward", "mj_sample_logits", "mj_sample_top_k", "mj_rmsnorm_workspace_bytes", "mj_rmsnorm_backward")
+           "mj_grpo_group_advantages", "mj_grpo_advantages", "mj_grpo_gae", "mj_rmsnorm_forward", "mj_sample_logits", "mj_sample_top_k", "mj_rmsnorm_workspace_bytes", "mj_rmsnorm_backward")
 
 KERNEL_NAMES = ("k_logits_stats", "k_finalize", "k_dz", "k_dhidden", "k_dhidden_reduce", "k_dw",
                 "k_reduce_loss")
@@ -64,6 +64,8 @@ def load() -> C.CDLL:
     lib.mj_grpo_profile_end.argtypes = [C.POINTER(C.c_double), C.POINTER(C.c_int)]
     i64, f32 = C.c_int64, C.c_float
     lib.mj_grpo_group_advantages.argtypes = [fp, ip, fp, i64, f32, vp]
+    lib.mj_grpo_advantages.argtypes = [C.c_int, fp, ip, fp, i64, f32, f32, C.c_int, f32, vp]
+    lib.mj_grpo_gae.argtypes = [fp, fp, fp, fp, fp, i64, i64, f32, f32, C.c_int, f32, f32, vp]
     lib.mj_sample_logits.argtypes = [vp, i64, vp, i64, fp, i64, i64, i64, i64, f32, vp]
     lib.mj_sample_top_k.argtypes = [fp, i64, i64, i64, C.c_int, f32, fp, ip, ip, fp, vp]
     lib.mj_rmsnorm_forward.argtypes = [vp, i64, fp, vp, i64, fp, i64, i64, f32, vp]

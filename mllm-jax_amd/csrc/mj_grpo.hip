@@ -428,14 +428,45 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
 
 }  // extern "C"
 
-extern "C" int mj_grpo_group_advantages(const float* rewards, const int32_t* group_ids, float* advantages, int64_t b,
-                                        float eps, void* stream) {
-  if (!rewards || !group_ids || !advantages) return fail(MJ_GRPO_ERR_NULL, "rewards/group_ids/advantages is NULL");
-  if (b <= 0 || b > (1 << 20)) return fail(MJ_GRPO_ERR_SHAPE, "batch must be in [1, 2^20] (got %lld)", (long long)b);
-  mj::k_group_advantages<<<(unsigned)((b + 255) / 256), 256, 0, (hipStream_t)stream>>>(rewards, group_ids, advantages,
-                                                                                         (int)b, eps);
-  return check_launch("k_group_advantages");
+extern "C" {
+
+int mj_grpo_advantages(int mode, const float* rewards, const int32_t* group_ids, float* advantages, int64_t b,
+                       float eps, float alpha, int whiten, float clip_range, void* stream) {
+  if (mode < mj::kAdvGrpo || mode > mj::kAdvDapo) return fail(MJ_GRPO_ERR_UNSUPPORTED, "unknown advantage mode %d", mode);
+  if (!rewards || !advantages || (mode != mj::kAdvGlobal && !group_ids))
+    return fail(MJ_GRPO_ERR_NULL, "rewards/group_ids/advantages is NULL");
+  if (b <= 0 || b > (1 << 16)) return fail(MJ_GRPO_ERR_SHAPE, "batch must be in [1, 65536] (got %lld)", (long long)b);
+  if (!(eps > 0.f)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "eps must be > 0");
+  if (mode == mj::kAdvDapo && !(alpha >= 0.f)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "alpha must be >= 0");
+  mj::AdvArgs a;
+  a.rewards = rewards; a.group_ids = group_ids; a.adv = advantages; a.b = (int)b; a.mode = mode; a.whiten = whiten;
+  a.eps = eps; a.alpha = alpha; a.clip = clip_range;
+  mj::k_advantages<<<1, 1024, 0, (hipStream_t)stream>>>(a);
+  return check_launch("k_advantages");
 }
+
+int mj_grpo_group_advantages(const float* rewards, const int32_t* group_ids, float* advantages, int64_t b, float eps,
+                             void* stream) {
+  return mj_grpo_advantages(mj::kAdvGrpo, rewards, group_ids, advantages, b, eps, 0.f, 0, 0.f, stream);
+}
+
+int mj_grpo_gae(const float* rewards, const float* values, const float* completion_mask, float* advantages,
+                float* returns, int64_t b, int64_t t, float gamma, float gae_lambda, int normalize, float eps,
+                float clip_range, void* stream) {
+  if (!rewards || !values || !completion_mask || !advantages || !returns) return fail(MJ_GRPO_ERR_NULL, "gae: NULL pointer argument");
+  if (b <= 0 || t <= 0 || b > (1 << 24) || t > (1 << 24) || b * t > (1ll << 31))
+    return fail(MJ_GRPO_ERR_SHAPE, "gae: bad shape b=%lld t=%lld", (long long)b, (long long)t);
+  mj::GaeArgs a;
+  a.rewards = rewards; a.values = values; a.mask = completion_mask; a.adv = advantages; a.ret = returns;
+  a.b = (int)b; a.t = (int)t; a.gamma = gamma; a.lambda = gae_lambda;
+  hipStream_t st = (hipStream_t)stream;
+  mj::k_gae_scan<<<(unsigned)((b + 255) / 256), 256, 0, st>>>(a);
+  if (normalize || clip_range > 0.f)
+    mj::k_gae_normalize<<<1, 1024, 0, st>>>(advantages, completion_mask, b * t, normalize, eps, clip_range);
+  return check_launch("gae kernels");
+}
+
+}  // extern "C"
 
 // ----------------------------------------------------------------------------- sampler
 extern "C" {

@@ -805,26 +805,135 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
 }
 
 // ----------------------------------------------------------------------------- advantages
-// Group-normalised advantages (plugins/training/advantage/grpo.py:28-52): per group id,
-// (r - mean) / (std + eps) with the population std.  B is a batch of sequences (hundreds), so
-// each thread simply walks the batch for its own element: sums in double in index order (what
-// np.bincount does), the remaining arithmetic in float like the NumPy original.
-__global__ __launch_bounds__(256) void k_group_advantages(const float* rewards, const int32_t* group_ids, float* adv,
-                                                          int b, float eps) {
+// Sequence-level advantage estimators (plugins/training/advantage/grpo.py:8-52 and
+// advantage/estimators.py:37-157).  B is a batch of sequences (hundreds to thousands): one
+// workgroup does everything, each thread walks the batch for its own samples; sums in double in
+// index order, the remaining arithmetic in float like the NumPy originals.
+enum AdvMode { kAdvGrpo = 0, kAdvGlobal = 1, kAdvRloo = 2, kAdvDapo = 3 };
+
+struct AdvArgs {
+  const float* rewards;
+  const int32_t* group_ids;   // unused by kAdvGlobal
+  float* adv;
+  int b, mode, whiten;        // whiten: kAdvRloo only
+  float eps, alpha, clip;     // clip <= 0: none
+};
+
+MJ_DEV void block_mean_std(const float* x, int n, double* sh, float& mean, float& stdv) {
+  // population mean and standard deviation over x[0..n), all threads get the result
+  const int t = threadIdx.x;
+  double a = 0.0;
+  for (int i = t; i < n; i += 1024) a += (double)x[i];
+  sh[t] = a;
+  __syncthreads();
+  for (int o = 512; o > 0; o >>= 1) { if (t < o) sh[t] += sh[t + o]; __syncthreads(); }
+  const double m = sh[0] / n;
+  __syncthreads();
+  double v = 0.0;
+  for (int i = t; i < n; i += 1024) { const double d = (double)x[i] - m; v += d * d; }
+  sh[t] = v;
+  __syncthreads();
+  for (int o = 512; o > 0; o >>= 1) { if (t < o) sh[t] += sh[t + o]; __syncthreads(); }
+  mean = (float)m;
+  stdv = (float)sqrt(sh[0] / n);
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(1024) void k_advantages(AdvArgs p) {
+  __shared__ double sh[1024];
+  float rmean = 0.f, rstd = 0.f;
+  if (p.mode == kAdvGlobal || p.mode == kAdvDapo) block_mean_std(p.rewards, p.b, sh, rmean, rstd);
+  for (int i = threadIdx.x; i < p.b; i += 1024) {
+    const float r = p.rewards[i];
+    float out;
+    if (p.mode == kAdvGlobal) {
+      out = (r - rmean) / (rstd + p.eps);                                   // estimators.py:52-55
+    } else {
+      const int gid = p.group_ids[i];
+      double sum = 0.0;
+      int cnt = 0;
+      for (int j = 0; j < p.b; ++j)
+        if (p.group_ids[j] == gid) { sum += (double)p.rewards[j]; ++cnt; }
+      const float gsum = (float)sum, count = fmaxf((float)cnt, 1.f);
+      if (p.mode == kAdvRloo) {                                             // estimators.py:88-97
+        const float loo = (gsum - r) / fmaxf((float)cnt - 1.f, 1.f);
+        out = r - (cnt > 1 ? loo : gsum / count);
+      } else {                                                              // grpo.py:40-51
+        const float mean = gsum / count;
+        double sq = 0.0;
+        for (int j = 0; j < p.b; ++j)
+          if (p.group_ids[j] == gid) { const float c = p.rewards[j] - mean; sq += (double)(c * c); }
+        out = (r - mean) / (sqrtf((float)sq / count) + p.eps);
+        if (p.mode == kAdvDapo) out += p.alpha * ((r - rmean) / (rstd + p.eps));   // estimators.py:131-133
+      }
+    }
+    p.adv[i] = out;
+  }
+  __syncthreads();
+  if (p.mode == kAdvRloo && p.whiten) {                                     // estimators.py:99-102
+    float m, sd;
+    block_mean_std(p.adv, p.b, sh, m, sd);
+    for (int i = threadIdx.x; i < p.b; i += 1024) p.adv[i] = (p.adv[i] - m) / (sd + p.eps);
+    __syncthreads();
+  }
+  if (p.clip > 0.f)
+    for (int i = threadIdx.x; i < p.b; i += 1024) p.adv[i] = fminf(fmaxf(p.adv[i], -p.clip), p.clip);
+}
+
+// Token-level GAE (advantage/estimators.py:160-240): the sequence reward sits on the last
+// completion token; one thread scans its sequence backwards.
+struct GaeArgs {
+  const float *rewards, *values, *mask;   // [B], [B,T], [B,T]
+  float *adv, *ret;                       // [B,T]
+  int b, t;
+  float gamma, lambda;
+};
+
+__global__ __launch_bounds__(256) void k_gae_scan(GaeArgs p) {
   const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= b) return;
-  const int gid = group_ids[i];
-  double sum = 0.0;
-  int cnt = 0;
-  for (int j = 0; j < b; ++j)
-    if (group_ids[j] == gid) { sum += (double)rewards[j]; ++cnt; }
-  const float count = fmaxf((float)cnt, 1.f);
-  const float mean = (float)sum / count;
-  double sq = 0.0;
-  for (int j = 0; j < b; ++j)
-    if (group_ids[j] == gid) { const float c = rewards[j] - mean; sq += (double)(c * c); }
-  const float var = (float)sq / count;
-  adv[i] = (rewards[i] - mean) / (sqrtf(var) + eps);
+  if (i >= p.b) return;
+  const float* v = p.values + (int64_t)i * p.t;
+  const float* m = p.mask + (int64_t)i * p.t;
+  int last = -1;
+  for (int k = 0; k < p.t; ++k) if (m[k] > 0.f) last = k;
+  float gae = 0.f, next_v = 0.f;
+  for (int k = p.t - 1; k >= 0; --k) {
+    const float rew = (k == last) ? p.rewards[i] : 0.f;
+    const float delta = rew + p.gamma * next_v - v[k];
+    gae = (delta + p.gamma * p.lambda * gae) * m[k];
+    p.adv[(int64_t)i * p.t + k] = gae;
+    p.ret[(int64_t)i * p.t + k] = gae + v[k];
+    next_v = v[k] * m[k];
+  }
+}
+
+// normalisation over the completion tokens (estimators.py:226-232) and the optional clip
+__global__ __launch_bounds__(1024) void k_gae_normalize(float* adv, const float* mask, int64_t n, int normalize,
+                                                        float eps, float clip) {
+  __shared__ double sh[1024];
+  __shared__ double cnt_sh[1024];
+  const int t = threadIdx.x;
+  if (normalize) {
+    double a = 0.0, c = 0.0;
+    for (int64_t i = t; i < n; i += 1024) if (mask[i] > 0.f) { a += (double)adv[i]; c += 1.0; }
+    sh[t] = a; cnt_sh[t] = c;
+    __syncthreads();
+    for (int o = 512; o > 0; o >>= 1) { if (t < o) { sh[t] += sh[t + o]; cnt_sh[t] += cnt_sh[t + o]; } __syncthreads(); }
+    const double cnt = cnt_sh[0], mean = cnt > 0 ? sh[0] / cnt : 0.0;
+    __syncthreads();
+    double v = 0.0;
+    for (int64_t i = t; i < n; i += 1024) if (mask[i] > 0.f) { const double d = (double)adv[i] - mean; v += d * d; }
+    sh[t] = v;
+    __syncthreads();
+    for (int o = 512; o > 0; o >>= 1) { if (t < o) sh[t] += sh[t + o]; __syncthreads(); }
+    if (cnt > 0) {
+      const float m = (float)mean, sd = (float)sqrt(sh[0] / cnt);
+      for (int64_t i = t; i < n; i += 1024) adv[i] = mask[i] > 0.f ? (adv[i] - m) / (sd + eps) : 0.f;
+    }
+    __syncthreads();
+  }
+  if (clip > 0.f)
+    for (int64_t i = t; i < n; i += 1024) adv[i] = fminf(fmaxf(adv[i], -clip), clip);
 }
 
 }  // namespace mj

@@ -11,6 +11,7 @@ reference's un-fused jnp loss:
   deprecated/MLLM_JAX/language/gemma/transformer.py:337-339 (final-logit softcap)
   plugins/training/update/train_step.py:15-24  (value_and_grad -> closed-form backward)
   plugins/training/advantage/grpo.py:28-52     (group-normalised advantages)
+  plugins/training/advantage/estimators.py     (global / RLOO / DAPO / REINFORCE++ / GAE)
   plugins/training/ppo/module.py:59-150        (actor-critic twin: policy + value + entropy bonus)
   plugins/sft/jax/sft_module.py:22-45          (masked cross-entropy)
   MLLM_JAX/language/llama/llama.py:426-452     (RMSNorm producing `hidden`)
@@ -272,6 +273,65 @@ def grpo_advantages(rewards, group_ids, eps=1e-4):
     c = r - mean[inv]
     std = np.sqrt(np.bincount(inv, weights=c * c, minlength=ng).astype(np.float32) / cnt)
     return (c / (std[inv] + float(eps))).astype(np.float32)
+
+
+def _group_index(group_ids):
+    return np.unique(np.asarray(group_ids).reshape(-1), return_inverse=True)[1]
+
+
+def global_normalized_advantages(rewards, eps=1e-4, clip_range=None):
+    """advantage/estimators.py:37-55."""
+    r = np.asarray(rewards, np.float32).reshape(-1)
+    a = ((r - np.float32(r.mean())) / (np.float32(r.std()) + np.float32(eps))).astype(np.float32)
+    return a if clip_range is None else np.clip(a, -clip_range, clip_range)
+
+
+def rloo_advantages(rewards, group_ids, eps=1e-4, whiten=True, clip_range=None):
+    """advantage/estimators.py:58-103: leave-one-out baseline inside each group (group mean for
+    singletons), optional whitening over the batch."""
+    r = np.asarray(rewards, np.float32).reshape(-1)
+    inv = _group_index(group_ids)
+    gsum = np.bincount(inv, weights=r).astype(np.float32)[inv]
+    cnt = np.bincount(inv).astype(np.float32)[inv]
+    base = np.where(cnt > 1, (gsum - r) / np.maximum(cnt - 1, 1), gsum / np.maximum(cnt, 1)).astype(np.float32)
+    a = (r - base).astype(np.float32)
+    if whiten:
+        a = ((a - np.float32(a.mean())) / (np.float32(a.std()) + np.float32(eps))).astype(np.float32)
+    return a if clip_range is None else np.clip(a, -clip_range, clip_range)
+
+
+def dapo_advantages(rewards, group_ids, eps=1e-4, alpha=0.2, clip_range=None):
+    """advantage/estimators.py:106-134."""
+    a = (grpo_advantages(rewards, group_ids, eps) + np.float32(alpha) * global_normalized_advantages(rewards, eps)).astype(np.float32)
+    return a if clip_range is None else np.clip(a, -clip_range, clip_range)
+
+
+def gae_advantages(rewards, values, completion_mask, gamma=1.0, gae_lambda=0.95, normalize=True, eps=1e-4,
+                   clip_range=None):
+    """advantage/estimators.py:160-240: (advantages, returns), both [B,T] float32."""
+    r = np.asarray(rewards, np.float32).reshape(-1)
+    v = np.asarray(values, np.float32)
+    m = np.asarray(completion_mask, np.float32)
+    b, t = v.shape
+    tok = np.zeros_like(m)
+    for i in range(b):
+        idx = np.nonzero(m[i] > 0)[0]
+        if idx.size:
+            tok[i, idx[-1]] = r[i]
+    adv = np.zeros_like(v)
+    gae = np.zeros(b, np.float32); nxt = np.zeros(b, np.float32)
+    for k in range(t - 1, -1, -1):
+        delta = tok[:, k] + np.float32(gamma) * nxt - v[:, k]
+        gae = ((delta + np.float32(gamma) * np.float32(gae_lambda) * gae) * m[:, k]).astype(np.float32)
+        adv[:, k] = gae
+        nxt = v[:, k] * m[:, k]
+    ret = (adv + v).astype(np.float32)
+    if normalize and (m > 0).any():
+        sel = adv[m > 0]
+        adv = np.where(m > 0, (adv - np.float32(sel.mean())) / (np.float32(sel.std()) + np.float32(eps)), 0.0).astype(np.float32)
+    if clip_range is not None:
+        adv = np.clip(adv, -clip_range, clip_range).astype(np.float32)
+    return adv, ret
 
 
 def sft_cross_entropy(hidden, lm_head, labels, valid, *, with_grads=True):

@@ -383,3 +383,38 @@ def test_top_k_sample_against_torch_topk_and_by_hand(rng):
     draws = np.array([O.top_k_sample(z, k=3, t=1.0, noise=g[i:i + 1])[0][0] for i in range(0, 20000, 10)])
     freq = np.bincount(draws, minlength=3) / len(draws)
     np.testing.assert_allclose(freq, [0.6, 0.3, 0.1], atol=0.04)
+
+
+# --------------------------------------------------------------------------- advantage estimators
+# The known answers below are the ones the reference's own tests hold
+# (tests/test_advantage_estimators.py:19-106): same inputs, same expected values.
+R5 = np.asarray([1.0, 2.0, 3.0, 10.0, 20.0], np.float32)
+G5 = np.asarray([0, 0, 0, 1, 1], np.int32)
+
+
+def test_advantage_estimators_reference_known_answers():
+    r4 = np.asarray([0.0, 1.0, 2.0, 3.0], np.float32)
+    np.testing.assert_allclose(O.global_normalized_advantages(r4, 1e-4), (r4 - r4.mean()) / (r4.std() + 1e-4), atol=1e-6)
+    out = O.global_normalized_advantages(np.asarray([-100.0, 0.0, 100.0], np.float32), 1e-6, clip_range=0.5)
+    assert (out <= 0.5).all() and (out >= -0.5).all()
+    np.testing.assert_allclose(O.rloo_advantages(R5, G5, eps=1e-6, whiten=False), [-1.5, 0.0, 1.5, -10.0, 10.0], atol=1e-6)
+    w = O.rloo_advantages(R5, G5, eps=1e-6, whiten=True)
+    assert abs(float(w.mean())) < 1e-5 and float(w.std()) > 0.5
+    np.testing.assert_allclose(O.dapo_advantages(R5, G5, 1e-4, 0.5),
+                               O.grpo_advantages(R5, G5, 1e-4) + 0.5 * O.global_normalized_advantages(R5, 1e-4), atol=1e-6)
+    one = np.ones((1, 3), np.float32)
+    adv, ret = O.gae_advantages([1.0], np.zeros((1, 3), np.float32), one, 1.0, 1.0, normalize=False, eps=1e-6)
+    np.testing.assert_allclose(adv, one, atol=1e-6); np.testing.assert_allclose(ret, one, atol=1e-6)
+    adv, _ = O.gae_advantages([1.0], np.zeros((1, 3), np.float32), np.asarray([[0.0, 1.0, 1.0]], np.float32), 1.0, 1.0,
+                              normalize=False, eps=1e-6)
+    np.testing.assert_allclose(adv, [[0.0, 1.0, 1.0]], atol=1e-6)
+
+
+def test_gae_by_hand_with_discount_and_values():
+    # one sequence, completion tokens 1..2, reward 2 on the last: delta_2 = 2 - v2, delta_1 = g*v2 - v1
+    v = np.asarray([[0.5, 0.2, -0.1, 0.9]], np.float32); m = np.asarray([[0, 1, 1, 0]], np.float32)
+    g, lam = 0.9, 0.8
+    adv, ret = O.gae_advantages([2.0], v, m, g, lam, normalize=False)
+    d2 = 2.0 - (-0.1); d1 = g * (-0.1) - 0.2
+    np.testing.assert_allclose(adv, [[0.0, d1 + g * lam * d2, d2, 0.0]], atol=1e-6)
+    np.testing.assert_allclose(ret, adv + v, atol=1e-7)
