@@ -353,7 +353,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
 
 extern "C" {
 
-int mj_grpo_version(void) { return 100; }
+int mj_grpo_version(void) { return 200; }
 
 const char* mj_grpo_last_error(void) { return g_err; }
 
