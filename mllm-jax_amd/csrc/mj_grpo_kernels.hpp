@@ -703,15 +703,130 @@ MJ_DEV uint32_t topk_key(float f) {   // larger float <=> larger key; -0 and +0 
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+MJ_DEV float topk_unkey(uint32_t key) {
+  return __uint_as_float((key & 0x80000000u) ? (key ^ 0x80000000u) : ~key);
+}
+
+constexpr int kTopKPool = 4096;
+
 __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
-  __shared__ uint32_t hist[256];
-  __shared__ uint32_t s_prefix, s_need, s_cnt, s_wave[16], s_base;
+  __shared__ uint32_t hist[4096];
+  __shared__ uint32_t pool_key[kTopKPool];
+  __shared__ int pool_idx[kTopKPool];
+  __shared__ uint32_t s_scan[1024];
+  __shared__ uint32_t s_prefix, s_need, s_cnt, s_pool, s_wave[16], s_base;
   __shared__ float c_val[kTopKMax], o_val[kTopKMax];
   __shared__ int c_idx[kTopKMax], o_idx[kTopKMax];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* row = p.logits + (int64_t)blockIdx.x * p.ld;
-  // the k-th largest key, most significant byte first
-  uint32_t prefix = 0, need = (uint32_t)p.k;   // `need` keys still to find among those matching `prefix`
+
+  // ---- fast path, two reads of the row: a 12-bit histogram finds the bin of the k-th largest
+  // key; a second read sends larger keys straight to the result and the bin's keys to an LDS pool,
+  // where the selection finishes.  A bin that overflows the pool (many near-equal logits) falls
+  // back to the byte-wise select below.
+  for (int b = tid; b < 4096; b += 1024) hist[b] = 0;
+  if (tid == 0) { s_cnt = 0; s_pool = 0; s_base = 0; }
+  __syncthreads();
+  for (int i = tid; i < p.V; i += 1024) atomicAdd(&hist[topk_key(row[i] * p.inv_t) >> 20], 1u);
+  __syncthreads();
+  {
+    // suffix sums over the bins, four bins per thread (thread t owns bins 4t .. 4t+3)
+    const uint32_t mine = hist[4 * tid] + hist[4 * tid + 1] + hist[4 * tid + 2] + hist[4 * tid + 3];
+    s_scan[tid] = mine;
+    __syncthreads();
+    for (int o = 1; o < 1024; o <<= 1) {
+      const uint32_t v = tid + o < 1024 ? s_scan[tid + o] : 0u;
+      __syncthreads();
+      s_scan[tid] += v;
+      __syncthreads();
+    }
+    const uint32_t incl = s_scan[tid], excl = incl - mine;       // keys in bins >= 4t, and in bins > 4t+3
+    if (excl < (uint32_t)p.k && incl >= (uint32_t)p.k) {         // exactly one thread
+      uint32_t acc = excl;
+      int bin = 4 * tid + 3;
+      for (; bin > 4 * tid; --bin) {
+        if (acc + hist[bin] >= (uint32_t)p.k) break;
+        acc += hist[bin];
+      }
+      s_prefix = (uint32_t)bin;            // 12-bit bin of the k-th largest
+      s_need = (uint32_t)p.k - acc;        // how many of that bin's keys belong to the top k
+    }
+    __syncthreads();
+  }
+  const uint32_t bin12 = s_prefix;
+  uint32_t need = s_need;
+  for (int i = tid; i < p.V; i += 1024) {
+    const float v = row[i] * p.inv_t;
+    const uint32_t key = topk_key(v), hi = key >> 20;
+    if (hi > bin12) {
+      const uint32_t slot = atomicAdd(&s_cnt, 1u);
+      c_val[slot] = v;
+      c_idx[slot] = i;
+    } else if (hi == bin12) {
+      const uint32_t slot = atomicAdd(&s_pool, 1u);
+      if (slot < (uint32_t)kTopKPool) { pool_key[slot] = key; pool_idx[slot] = i; }
+    }
+  }
+  __syncthreads();
+  const uint32_t pooled = s_pool;
+  if (pooled <= (uint32_t)kTopKPool) {
+    // the low 20 bits of the k-th largest key, 10 bits at a time, over the pool
+    uint32_t prefix = bin12 << 20;
+    for (int pass = 0; pass < 2; ++pass) {
+      const int shift = 10 - 10 * pass;
+      hist[tid] = 0;
+      __syncthreads();
+      const uint32_t hi_mask = 0xffffffffu << (shift + 10);
+      for (uint32_t q = tid; q < pooled; q += 1024) {
+        const uint32_t key = pool_key[q];
+        if ((key & hi_mask) == prefix) atomicAdd(&hist[(key >> shift) & 1023u], 1u);
+      }
+      __syncthreads();
+      {
+        // suffix sums over the 1024 bins, one per thread: the bin where they cross `need`
+        const uint32_t mine = hist[tid];
+        s_scan[tid] = mine;
+        __syncthreads();
+        for (int o = 1; o < 1024; o <<= 1) {
+          const uint32_t v = tid + o < 1024 ? s_scan[tid + o] : 0u;
+          __syncthreads();
+          s_scan[tid] += v;
+          __syncthreads();
+        }
+        const uint32_t incl = s_scan[tid], excl = incl - mine;
+        if (excl < need && incl >= need) {
+          s_prefix = prefix | ((uint32_t)tid << shift);
+          s_need = need - excl;
+        }
+        __syncthreads();
+      }
+      prefix = s_prefix;
+      need = s_need;
+      __syncthreads();
+    }
+    // pool keys above the threshold in any order; equal keys by ascending index
+    const uint32_t above = s_cnt;
+    __syncthreads();
+    if (tid == 0) s_cnt = above + need;            // slots [above, above + need) belong to the equal keys
+    __syncthreads();
+    for (uint32_t q = tid; q < pooled; q += 1024) {
+      const uint32_t key = pool_key[q];
+      if (key > prefix) {
+        const uint32_t slot = atomicAdd(&s_cnt, 1u);
+        c_val[slot] = topk_unkey(key);
+        c_idx[slot] = pool_idx[q];
+      } else if (key == prefix) {
+        const int ix = pool_idx[q];
+        uint32_t rank = 0;
+        for (uint32_t r = 0; r < pooled; ++r) rank += (pool_key[r] == prefix && pool_idx[r] < ix) ? 1u : 0u;
+        if (rank < need) { c_val[above + rank] = topk_unkey(key); c_idx[above + rank] = ix; }
+      }
+    }
+    __syncthreads();
+  } else {
+  // ---- fallback: the k-th largest key, most significant byte first, over the whole row
+  uint32_t prefix = 0;
+  need = (uint32_t)p.k;   // `need` keys still to find among those matching `prefix`
   for (int pass = 0; pass < 4; ++pass) {
     const int shift = 24 - 8 * pass;
     if (tid < 256) hist[tid] = 0;
@@ -773,6 +888,7 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
       s_base = t;
     }
     __syncthreads();
+  }
   }
   // order the k candidates: value descending, index ascending
   if (tid < p.k) {

@@ -76,3 +76,20 @@ def test_greedy_generator_draws_and_fused_step():
     assert int(M.top_k_sampling_batched(gen, peaked, k=50, t=1.0)[0]) == 123
     with pytest.raises(M._lib.MjGrpoError):
         M.top_k_sampling_batched(None, logits, k=65)
+
+
+def test_near_equal_logits_overflow_the_pool_and_take_the_slow_path():
+    # more than 4096 logits share the 12 leading key bits of the k-th largest: the byte-wise select runs
+    import mllm_jax_amd as M
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(2)
+    x = np.full((4, 30000), 1.5, np.float32)
+    x[1] += (rng.random(30000) * 1e-3).astype(np.float32)       # all inside one 12-bit bin, distinct low bits
+    x[2, ::7] = 9.0                                             # 4286 equal maxima: ties beyond k
+    x[3] = rng.integers(0, 3, 30000).astype(np.float32)         # three values
+    noise = rng.gumbel(size=(4, 50)).astype(np.float32)
+    tok, idx, val = M.top_k_sampling_batched(torch.tensor(noise), torch.tensor(x, device=dev), k=50, t=1.0, return_top_k=True)
+    rt, ri, rv = O.top_k_sample(x, k=50, t=1.0, noise=noise)
+    np.testing.assert_array_equal(idx.cpu().numpy(), ri)
+    np.testing.assert_array_equal(val.cpu().numpy(), rv)
+    np.testing.assert_array_equal(tok.cpu().numpy(), rt)
