@@ -514,7 +514,7 @@ namespace {
 constexpr int kNormMaxH = 8192;
 int norm_grid(int64_t n) {   // workgroups of the backward: enough to fill the GPU, each walks rows with this stride
   const int64_t blocks = (n + 3) / 4;
-  return (int)(blocks < 1024 ? blocks : 1024);
+  return (int)(blocks < 512 ? blocks : 512);
 }
 int norm_check(int64_t n, int64_t h, std::initializer_list<int64_t> lds, std::initializer_list<const void*> ptrs) {
   if (n <= 0 || h <= 0 || n > (1ll << 30)) return fail(MJ_GRPO_ERR_SHAPE, "rmsnorm: n and h must be positive (got %lld, %lld)", (long long)n, (long long)h);
@@ -579,7 +579,7 @@ int mj_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x, int64_t ld
     mj::k_rmsnorm_bwd<16><<<grid, 256, lds, st>>>(a);
   }
   if ((rc = check_launch("k_rmsnorm_bwd"))) return rc;
-  mj::k_rmsnorm_dscale<<<(unsigned)((h + 255) / 256), 256, 0, st>>>((const float*)workspace, grid, (int)h, dscale,
+  mj::k_rmsnorm_dscale<<<(unsigned)((h + 63) / 64), 256, 0, st>>>((const float*)workspace, grid, (int)h, dscale,
                                                                   accumulate_dscale);
   return check_launch("k_rmsnorm_dscale");
 }

@@ -179,14 +179,31 @@ __global__ __launch_bounds__(256) void k_rmsnorm_bwd(NormBwdArgs p) {
   }
 }
 
-// dscale[h] (+)= sum over partial rows, fixed order
+// dscale[h] (+)= sum over partial rows, fixed order.  Block = 64 columns x 4 row lanes; lane r
+// adds the partial rows r, r+4, ... (eight loads in flight), the four lanes are added through LDS.
 __global__ __launch_bounds__(256) void k_rmsnorm_dscale(const float* part, int parts, int H, float* dscale,
                                                         int accumulate) {
-  const int h = blockIdx.x * 256 + threadIdx.x;
-  if (h >= H) return;
+  __shared__ float sh[3][64];
+  const int cx = threadIdx.x & 63, ry = threadIdx.x >> 6;
+  const int h = blockIdx.x * 64 + cx;
   float a = 0.f;
-  for (int q = 0; q < parts; ++q) a += part[(int64_t)q * H + h];
-  dscale[h] = accumulate ? dscale[h] + a : a;
+  if (h < H) {
+    int q = ry;
+    for (; q + 28 < parts; q += 32) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = part[(int64_t)(q + 4 * u) * H + h];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) a += v[u];
+    }
+    for (; q < parts; q += 4) a += part[(int64_t)q * H + h];
+  }
+  if (ry > 0) sh[ry - 1][cx] = a;
+  __syncthreads();
+  if (ry == 0 && h < H) {
+    a = ((a + sh[0][cx]) + sh[1][cx]) + sh[2][cx];
+    dscale[h] = accumulate ? dscale[h] + a : a;
+  }
 }
 
 }  // namespace mj
