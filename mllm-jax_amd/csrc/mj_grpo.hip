@@ -275,7 +275,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       f.ent_coef = d->entropy_coef; f.inv_ent_cnt = d->inv_entropy_count; f.eterm = eterm + c0;
       f.ge = bonus ? ge : nullptr; f.hent = bonus ? hent : nullptr;
       Timed t(MJ_GRPO_K_FINALIZE, st);
-      mj::k_finalize<<<n_pad / 64, 256, 0, st>>>(f);
+      mj::k_finalize<<<n_pad / 64, 64 * mj::kFinSlices, 0, st>>>(f);
     } else {
       Timed t(MJ_GRPO_K_FINALIZE, st);
       mj::k_coeff_from_saved<<<(n_pad + 255) / 256, 256, 0, st>>>(

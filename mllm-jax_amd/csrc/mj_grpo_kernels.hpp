@@ -224,15 +224,16 @@ struct FinalizeArgs {
   float *ge, *hent;            // [n_pad] coef*mask*inv_ent_cnt*gscale and H_t, or null (no bonus / forward only)
 };
 
-// block = (64 tokens) x (4 slices of the partial list)
-__global__ __launch_bounds__(256) void k_finalize(FinalizeArgs p) {
-  __shared__ float sm[4][64], sl[4][64], ss[4][64], st[4][64];
+// block = (64 tokens) x (kFinSlices slices of the partial list)
+constexpr int kFinSlices = 16;
+__global__ __launch_bounds__(64 * kFinSlices) void k_finalize(FinalizeArgs p) {
+  __shared__ float sm[kFinSlices][64], sl[kFinSlices][64], ss[kFinSlices][64], st[kFinSlices][64];
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int t = blockIdx.x * 64 + tx;
   const bool tempered = p.inv_t != 1.f;   // then s and lt are sums under softmax(z / T)
   float m = kNegBig, l = 0.f, s = 0.f, lt = 0.f;
   if (t < p.n) {
-    for (int q = ty; q < p.parts; q += 4) {
+    for (int q = ty; q < p.parts; q += kFinSlices) {
       const int64_t o = (int64_t)q * p.ld_p + t;
       const float mq = p.pm[o], lq = p.pl[o], sq = p.ps[o];
       const float mn = fmaxf(m, mq);
@@ -256,10 +257,12 @@ __global__ __launch_bounds__(256) void k_finalize(FinalizeArgs p) {
     if (p.ge != nullptr && t < p.n_pad) p.ge[t] = 0.f;
     return;
   }
-  float M = fmaxf(fmaxf(sm[0][tx], sm[1][tx]), fmaxf(sm[2][tx], sm[3][tx]));
+  float M = sm[0][tx];
+#pragma unroll
+  for (int i = 1; i < kFinSlices; ++i) M = fmaxf(M, sm[i][tx]);
   float L = 0.f, S = 0.f, LT = 0.f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < kFinSlices; ++i) {
     const float w = __expf(sm[i][tx] - M);
     const float wt = tempered ? __expf((sm[i][tx] - M) * p.inv_t) : w;
     L += sl[i][tx] * w;
