@@ -145,14 +145,20 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
 
 bool misaligned(const void* p) { return ((uintptr_t)p & 15u) != 0; }
 
+// Raises the dynamic LDS limit of a tile kernel (128 KB > the 64 KB default) once per device and
+// thread; the attribute belongs to the function on the current device.
 template <typename K>
 int enable_lds(K kernel) {
-  static thread_local const void* done[8] = {};
-  for (auto& d : done) if (d == (const void*)kernel) return MJ_GRPO_OK;
-  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     mj::GemmTN<BM, BN>::kLdsBytes);
+  struct Done { const void* fn; int dev; };
+  static thread_local Done done[32] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+  for (auto& d : done) if (d.fn == (const void*)kernel && d.dev == dev) return MJ_GRPO_OK;
+  e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                          mj::GemmTN<BM, BN>::kLdsBytes);
   if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-  for (auto& d : done) if (d == nullptr) { d = (const void*)kernel; break; }
+  for (auto& d : done) if (d.fn == nullptr) { d.fn = (const void*)kernel; d.dev = dev; break; }
   return MJ_GRPO_OK;
 }
 
@@ -570,11 +576,13 @@ int mj_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x, int64_t ld
   if (h <= 4096) {
     mj::k_rmsnorm_bwd<8><<<grid, 256, lds, st>>>(a);
   } else {
-    static thread_local bool raised = false;
-    if (!raised) {
+    static thread_local int raised_dev = -1;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipGetDevice failed");
+    if (raised_dev != dev) {
       hipError_t e = hipFuncSetAttribute((const void*)mj::k_rmsnorm_bwd<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * kNormMaxH * 4);
       if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-      raised = true;
+      raised_dev = dev;
     }
     mj::k_rmsnorm_bwd<16><<<grid, 256, lds, st>>>(a);
   }
