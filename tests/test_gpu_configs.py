@@ -143,3 +143,24 @@ def test_config3_full_size_runs_and_is_consistent():
     assert rs <= 1e-3 * dw.double().abs().sum(-1).max().item()
     M.release_workspaces()
     torch.cuda.empty_cache()
+
+
+def test_config3_full_size_skip_masked_equals_dense():
+    """Same full-size shape (two chunks of 16384 tokens): leaving the masked tokens out of the backward
+    products changes neither the forward outputs nor d_hidden (bit for bit) and d_lm_head only by
+    summation order."""
+    M, cfg, kw, wl = _make(3)
+    args = (wl["hidden"], wl["lm_head"], wl["target_ids"], wl["old_logps"], wl["advantages"], wl["mask"])
+    opts = dict(total_valid_token_count=wl["total_valid_token_count"], seq_shape=wl["seq_shape"],
+                return_token_entropy=True, **kw)
+    met_d, (dh_d, dw_d) = M.grpo_loss_value_and_grad(*args, **opts)
+    dh_d, dw_d = dh_d.clone(), dw_d.clone()
+    met_s, (dh_s, dw_s) = M.grpo_loss_value_and_grad(*args, skip_masked=True, **opts)
+    torch.cuda.synchronize()
+    assert torch.equal(met_d["per_token_logps"], met_s["per_token_logps"])
+    assert torch.equal(met_d["token_entropy"], met_s["token_entropy"])
+    assert abs(float(met_d["loss"]) - float(met_s["loss"])) <= 1e-5 * abs(float(met_d["loss"]))
+    assert torch.equal(dh_d, dh_s)
+    assert _rel(dw_s, dw_d) <= 1e-3
+    M.release_workspaces()
+    torch.cuda.empty_cache()
