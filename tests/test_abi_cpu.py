@@ -150,3 +150,46 @@ def test_skip_masked_flag_enlarges_the_workspace(lib):
     n, h = d.n_tokens, d.hidden
     assert fwd1 >= fwd0 + n * h * 2 + n * 4 * 10          # slot-order hidden copy, permutation, per-token copies
     assert both1 - fwd1 >= both0 - fwd0 + n * h * 2       # slot-order d_hidden
+
+
+def test_headers_are_plain_c_and_the_library_links_from_c(lib, tmp_path):
+    """include/*.h must compile as C99 (no C++-isms, no torch types) and a C program must be able to
+    call the library through them: version, a rejected descriptor, the error text."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("gcc not available")
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include "mj_grpo.h"
+#include "mj_norm.h"
+#include "mj_sample.h"
+int main(void) {
+  MjGrpoDesc d;
+  size_t fwd = 0, both = 0;
+  memset(&d, 0, sizeof d);
+  d.n_tokens = 64; d.hidden = 64; d.vocab = 500; d.ld_hidden = 64; d.ld_w = 500;   /* vocab not a multiple of 8 */
+  d.temperature = 1.0f; d.inv_total_valid_tokens = 1.0f; d.grad_loss_scale = 1.0f;
+  if (mj_grpo_version() < 100) return 1;
+  if (mj_grpo_workspace_bytes(&d, &fwd, &both) != MJ_GRPO_ERR_ALIGN) return 2;
+  if (strstr(mj_grpo_last_error(), "multiples of 8") == NULL) return 3;
+  d.vocab = 512; d.ld_w = 512;
+  if (mj_grpo_workspace_bytes(&d, &fwd, &both) != MJ_GRPO_OK || both <= fwd) return 4;
+  if (mj_rmsnorm_workspace_bytes(8, 60, &fwd) != MJ_GRPO_ERR_ALIGN) return 5;
+  if (mj_sample_top_k(NULL, 512, 4, 512, 50, 1.0f, NULL, NULL, NULL, NULL, NULL) != MJ_GRPO_ERR_NULL) return 6;
+  printf("sizeof(MjGrpoDesc)=%zu\n", sizeof(MjGrpoDesc));
+  return 0;
+}
+''')
+    exe = tmp_path / "abi"
+    libdir = os.path.dirname(lib.LIB_PATH)
+    cmd = [gcc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+           "-L", libdir, "-l:libmj_grpo.so", "-Wl,-rpath," + libdir]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+    run = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert run.returncode == 0, (run.returncode, run.stdout, run.stderr)
+    assert "sizeof(MjGrpoDesc)=88" in run.stdout
