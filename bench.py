@@ -62,6 +62,67 @@ def _vendor_gemm(torch, hidden, w, mask, n, h, v, reps=5):
     return out
 
 
+class _SmiSampler:
+    """Polls `rocm-smi -P -c -t --json` in a thread while the timed loop runs (power, shader clock and
+    temperature as the driver reports them); the GPU work is not touched."""
+
+    def __init__(self, period_s=0.2):
+        import threading
+        self.period, self.samples, self._stop = period_s, [], threading.Event()
+        self._thread = threading.Thread(target=self._run, daemon=True)
+
+    def _run(self):
+        import re
+        import subprocess
+        while not self._stop.is_set():
+            try:
+                out = subprocess.run(["rocm-smi", "-P", "-c", "-t", "--json"], capture_output=True, text=True,
+                                     timeout=10).stdout
+                card = next(iter(json.loads(out).values()))
+                rec = {}
+                for k, v in card.items():
+                    m = re.search(r"[-+]?\d+(\.\d+)?", str(v))
+                    if not m:
+                        continue
+                    kl = k.lower()
+                    if "power" in kl and "max" not in kl:
+                        rec["power_w"] = float(m.group())
+                    elif kl.startswith("sclk"):
+                        rec["sclk_mhz"] = float(m.group())
+                    elif "junction" in kl:
+                        rec["junction_c"] = float(m.group())
+                if rec:
+                    rec["t"] = round(time.perf_counter(), 3)
+                    self.samples.append(rec)
+            except Exception as e:      # the sampler must never break the benchmark
+                self.samples.append({"error": repr(e)[:80]})
+                break
+            self._stop.wait(self.period)
+
+    def __enter__(self):
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        self._thread.join(timeout=15)
+
+    def summary(self, t0, t1):
+        inside = [r for r in self.samples if "t" in r and t0 + 0.3 <= r["t"] <= t1]
+        out = {"samples_in_timed_loop": len(inside), "samples_total": len(self.samples)}
+        for key in ("power_w", "sclk_mhz", "junction_c"):
+            vals = sorted(r[key] for r in inside if key in r)
+            if vals:
+                out[key] = {"min": vals[0], "median": vals[len(vals) // 2], "max": vals[-1]}
+        idle = [r for r in self.samples if "t" in r and r["t"] < t0 - 0.05]
+        if idle and "power_w" in idle[0]:
+            out["before_loop"] = {k: idle[-1].get(k) for k in ("power_w", "sclk_mhz", "junction_c")}
+        errs = [r["error"] for r in self.samples if "error" in r]
+        if errs:
+            out["error"] = errs[0]
+        return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -69,6 +130,13 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (default 2)")
     ap.add_argument("--chunk-tokens", type=int, default=0)
+    ap.add_argument("--dhidden-splits", type=int, default=0, help="vocab splits of the d_hidden product (0 = library's choice)")
+    ap.add_argument("--pad-w", type=int, default=0, help="extra elements in the row pitch of lm_head (ld_w = vocab + this)")
+    ap.add_argument("--smi", action="store_true",
+                    help="sample power / shader clock / temperature with rocm-smi during the timed loop (use >= 50 steps)")
+    ap.add_argument("--zero-operands", action="store_true",
+                    help="time the same launches with all-zero hidden and lm_head (MFMA power depends on the operand "
+                         "data; the loss value is then meaningless)")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-masked", action="store_true",
@@ -98,7 +166,7 @@ def main() -> int:
     dev = torch.device("cuda:0")
     cfg = M.CONFIGS[args.config]
     kw = dict(epsilon_low=cfg.eps_low, epsilon_high=cfg.eps_high, final_logit_softcap=cfg.softcap,
-              chunk_tokens=args.chunk_tokens or None)
+              chunk_tokens=args.chunk_tokens or None, dhidden_splits=args.dhidden_splits)
 
     def logp_fn(wl):
         with torch.no_grad():
@@ -108,7 +176,10 @@ def main() -> int:
 
     wl = M.make_workload(cfg, dev, 20250 + args.config, logp_fn=logp_fn)
     n, h, v = cfg.tokens, cfg.hidden, cfg.vocab
-    d_w = torch.empty(h, v, dtype=torch.float32, device=dev)
+    if args.pad_w:
+        wide = torch.zeros(h, v + args.pad_w, dtype=torch.bfloat16, device=dev)
+        wide[:, :v] = wl["lm_head"]
+        wl["lm_head"] = wide[:, :v]
 
     def step(skip_masked=args.skip_masked):
         return M.grpo_loss_value_and_grad(
@@ -116,6 +187,9 @@ def main() -> int:
             total_valid_token_count=wl["total_valid_token_count"], seq_shape=wl["seq_shape"],
             return_token_entropy=cfg.token_entropy, skip_masked=skip_masked, **kw)
 
+    if args.zero_operands:
+        wl["hidden"].zero_()
+        wl["lm_head"].zero_()
     if args.copy_calibration_mib:
         src = torch.empty(args.copy_calibration_mib << 20, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
@@ -126,14 +200,20 @@ def main() -> int:
         step()
     torch.cuda.synchronize()
     _lib.profile_begin(64 * max(args.steps, 1))
+    sampler = _SmiSampler() if args.smi else None
+    if sampler:
+        sampler.__enter__()
+        time.sleep(1.0)                 # a few idle samples first
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         metrics, grads = step()
     torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    t_end = time.perf_counter()
+    dt = t_end - t0
+    if sampler:
+        sampler.__exit__()
     prof = _lib.profile_end()
-    del d_w
 
     ms_per_step = dt / args.steps * 1e3
     tokens_per_s = n * args.steps / dt
@@ -160,6 +240,7 @@ def main() -> int:
         "config": {"workload": f"BASELINE configs[{args.config}] {cfg.name}: fused GRPO loss fwd+bwd, "
                                f"{n} tokens x hidden {h} x vocab {v}", "tokens": n, "hidden": h, "vocab": v,
                    "chunk_tokens": args.chunk_tokens or min(16384, n), "softcap": cfg.softcap,
+                   "ld_w": v + args.pad_w, "dhidden_splits": args.dhidden_splits or "auto",
                    "eps": [cfg.eps_low, cfg.eps_high]},
         "pct_bf16_mfma_peak": round(100.0 * mfu, 2),
         "algorithmic_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 1),
@@ -168,6 +249,10 @@ def main() -> int:
         "kernel_ms_per_step": {k: round(v_[0] / args.steps, 3) for k, v_ in prof.items()},
     }
 
+    if sampler:
+        line["smi"] = sampler.summary(t0, t_end)
+    if args.zero_operands:
+        line["config"]["operands"] = "all-zero hidden and lm_head"
     line["config"]["skip_masked"] = bool(args.skip_masked)
     if not args.skip_masked and not args.no_skip_masked_extra:
         # Not the headline: the same step with tokens that cannot carry a gradient (mask 0, advantage 0)

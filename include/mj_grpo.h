@@ -16,6 +16,8 @@
  * (train_modules/__init__.py:118-125).  hidden[N, ld_hidden] bf16 row-major,
  * lm_head[H, ld_w] bf16 row-major (Flax Dense kernel layout [in, out],
  * MLLM_JAX/language/llama/llama.py:889), targets[N] int32 in [0, V),
+ * (ids outside are clamped to the nearest valid id, the same way in both passes, without a
+ * host check; the reference's jnp.take_along_axis wraps negative ids and yields NaN past V),
  * old_logp[N] f32 or NULL (NULL = on-policy, ratio == 1, train_modules/__init__.py:161-165),
  * advantages[N] f32 (the reference's [B] broadcast per token, :173), mask[N] f32 in {0,1}.
  * Requirements: H % 8 == 0, V % 8 == 0, ld_hidden % 8 == 0, ld_w % 8 == 0,
@@ -70,7 +72,8 @@ typedef struct MjGrpoDesc {
   float inv_total_valid_tokens; /* 1 / total_valid_token_count (:179-180) */
   float grad_loss_scale; /* upstream d(loss); 1 for a terminal loss */
   uint32_t flags;
-  uint32_t reserved;
+  uint32_t dhidden_splits; /* pieces the vocab sum of the d_hidden product is cut into (fp32 partial sums,
+                            added in fixed order); 0 = chosen by the library, at most 32 */
   float entropy_coef;    /* PPOActorCriticModule.entropy_coef (plugins/training/ppo/module.py:140):
                             the loss becomes policy_loss - entropy_coef * entropy; 0 = GRPO */
   float inv_entropy_count; /* 1 / (sum(mask) + 1e-8), the normaliser of that entropy (:79); 0 = unused */

@@ -29,7 +29,7 @@ class MjGrpoDesc(C.Structure):
         ("ld_hidden", C.c_int64), ("ld_w", C.c_int64), ("chunk_tokens", C.c_int64),
         ("eps_low", C.c_float), ("eps_high", C.c_float), ("temperature", C.c_float),
         ("softcap", C.c_float), ("inv_total_valid_tokens", C.c_float), ("grad_loss_scale", C.c_float),
-        ("flags", C.c_uint32), ("reserved", C.c_uint32),
+        ("flags", C.c_uint32), ("dhidden_splits", C.c_uint32),
         ("entropy_coef", C.c_float), ("inv_entropy_count", C.c_float),
     ]
 

@@ -9,6 +9,7 @@
 #include <stdio.h>
 
 #include <initializer_list>
+#include <new>
 
 #include "mj_grpo_kernels.hpp"
 #include "mj_norm_kernels.hpp"
@@ -112,7 +113,8 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   p->n_pad = rup(chunk, 256);
   p->ld_z = p->n_pad;
   p->parts = 2 * ((p->V + BM - 1) / BM);
-  p->dh_splits = pick_splits((p->n_pad / BM) * ((p->H + BN - 1) / BN));
+  if (d->dhidden_splits > 32) return fail(MJ_GRPO_ERR_SHAPE, "dhidden_splits must be <= 32 (got %u)", d->dhidden_splits);
+  p->dh_splits = d->dhidden_splits ? (int)d->dhidden_splits : pick_splits((p->n_pad / BM) * ((p->H + BN - 1) / BN));
   p->dh_k_per_split = rup((p->V + p->dh_splits - 1) / p->dh_splits, 64);
   size_t o = 0;
   auto take = [&](size_t bytes) { size_t at = o; o = (size_t)rup((int64_t)(o + bytes), 256); return at; };
@@ -366,11 +368,17 @@ const char* mj_grpo_last_error(void) { return g_err; }
 int mj_grpo_profile_begin(int max_launches) {
   if (g_prof.on) return fail(MJ_GRPO_ERR_UNSUPPORTED, "profiling already on");
   if (max_launches <= 0 || max_launches > (1 << 16)) return fail(MJ_GRPO_ERR_SHAPE, "max_launches out of range");
-  g_prof.ev = new hipEvent_t[2 * (size_t)max_launches];
-  g_prof.kid = new int[max_launches];
-  for (int i = 0; i < 2 * max_launches; ++i) {
-    hipError_t e = hipEventCreate(&g_prof.ev[i]);
-    if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipEventCreate: %s", hipGetErrorString(e));
+  g_prof.ev = new (std::nothrow) hipEvent_t[2 * (size_t)max_launches];
+  g_prof.kid = new (std::nothrow) int[max_launches];
+  hipError_t e = (g_prof.ev && g_prof.kid) ? hipSuccess : hipErrorOutOfMemory;
+  int made = 0;
+  for (; e == hipSuccess && made < 2 * max_launches; ++made) e = hipEventCreate(&g_prof.ev[made]);
+  if (e != hipSuccess) {   // undo the partial set-up: nothing stays allocated after a failure
+    for (int i = 0; i + 1 < made; ++i) (void)hipEventDestroy(g_prof.ev[i]);
+    delete[] g_prof.ev;
+    delete[] g_prof.kid;
+    g_prof = Profiler();
+    return fail(MJ_GRPO_ERR_HIP, "profile set-up: %s", hipGetErrorString(e));
   }
   g_prof.cap = max_launches;
   g_prof.used = 0;
@@ -507,7 +515,7 @@ int mj_sample_top_k(const float* logits, int64_t ld_logits, int64_t b, int64_t v
   if (k < 1 || k > mj::kTopKMax || k > vocab) return fail(MJ_GRPO_ERR_UNSUPPORTED, "sample_top_k: k must be in [1, min(%d, vocab)] (got %d)", mj::kTopKMax, k);
   if (!(temperature > 0.f) || !isfinite(temperature)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "sample_top_k: temperature must be > 0");
   mj::TopKArgs a;
-  a.logits = logits; a.ld = ld_logits; a.V = (int)vocab; a.k = k; a.inv_t = 1.f / temperature; a.noise = noise;
+  a.logits = logits; a.ld = ld_logits; a.V = (int)vocab; a.k = k; a.t = temperature; a.noise = noise;
   a.token = token; a.top_idx = top_idx; a.top_val = top_val;
   mj::k_topk_sample<<<(unsigned)b, 1024, 0, (hipStream_t)stream>>>(a);
   return check_launch("k_topk_sample");

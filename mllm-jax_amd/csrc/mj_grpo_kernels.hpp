@@ -61,6 +61,9 @@ MJ_DEV f32x4 load_b128(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
   return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
 
+// Target ids outside [0, V) select the nearest valid id, in the forward and the backward alike.
+MJ_DEV int clamp_target(int y, int V) { return min(max(y, 0), V - 1); }
+
 // Tokens of a chunk that take part in the backward pass, rounded up to whole 256-token tiles:
 // all n_pad of them, or -- when the caller compacted the tokens that carry a gradient to the
 // front -- those up to the device-side count.
@@ -180,8 +183,7 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
     // The sampled token's logit: exactly one lane of one tile holds it.  Few wavefronts have a
     // hit at all (32 tokens x 128 rows out of V), so the register search sits behind a vote.
     {
-      int y = col < p.n ? p.targets[col] : -1;
-      y = y >= p.V ? p.V - 1 : y;
+      const int y = col < p.n ? clamp_target(p.targets[col], p.V) : -1;
       const int d = y - vwave;                       // row inside the wavefront's 128
       const bool hit = y >= 0 && d >= 0 && d < G::WM && ((d >> 2) & 1) == lhi;
       if (__any(hit)) {
@@ -383,7 +385,7 @@ __global__ __launch_bounds__(256) void k_dz(DzArgs p) {
     const bool in = t < p.n;
     lse[i] = in ? p.lse[t] * kLog2e : 0.f;
     g[i] = in ? p.g[t] : 0.f;
-    y[i] = in ? p.targets[t] : -1;
+    y[i] = in ? clamp_target(p.targets[t], p.V) : -1;
     ge[i] = (bonus && in) ? p.ge[t] : 0.f;
     hent[i] = (bonus && in) ? p.hent[t] : 0.f;
   }
@@ -694,7 +696,7 @@ struct TopKArgs {
   const float* logits;   // [b, ld]
   int64_t ld;
   int V, k;
-  float inv_t;
+  float t;                // temperature: keys are logits / t (MLLM_JAX/sample/sanple_utils.py:37)
   const float* noise;    // [b, k] or null (greedy: the largest)
   int32_t* token;        // [b]
   int32_t* top_idx;      // [b, k] or null
@@ -730,7 +732,7 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
   for (int b = tid; b < 4096; b += 1024) hist[b] = 0;
   if (tid == 0) { s_cnt = 0; s_pool = 0; s_base = 0; }
   __syncthreads();
-  for (int i = tid; i < p.V; i += 1024) atomicAdd(&hist[topk_key(row[i] * p.inv_t) >> 20], 1u);
+  for (int i = tid; i < p.V; i += 1024) atomicAdd(&hist[topk_key(row[i] / p.t) >> 20], 1u);
   __syncthreads();
   {
     // suffix sums over the bins, four bins per thread (thread t owns bins 4t .. 4t+3)
@@ -759,7 +761,7 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
   const uint32_t bin12 = s_prefix;
   uint32_t need = s_need;
   for (int i = tid; i < p.V; i += 1024) {
-    const float v = row[i] * p.inv_t;
+    const float v = row[i] / p.t;
     const uint32_t key = topk_key(v), hi = key >> 20;
     if (hi > bin12) {
       const uint32_t slot = atomicAdd(&s_cnt, 1u);
@@ -836,7 +838,7 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
     __syncthreads();
     const uint32_t hi_mask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
     for (int i = tid; i < p.V; i += 1024) {
-      const uint32_t key = topk_key(row[i] * p.inv_t);
+      const uint32_t key = topk_key(row[i] / p.t);
       if ((key & hi_mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
     }
     __syncthreads();
@@ -859,7 +861,7 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
   if (tid == 0) { s_cnt = 0; s_base = 0; }
   __syncthreads();
   for (int i = tid; i < p.V; i += 1024) {
-    const float v = row[i] * p.inv_t;
+    const float v = row[i] / p.t;
     if (topk_key(v) > prefix) {
       const uint32_t slot = atomicAdd(&s_cnt, 1u);
       c_val[slot] = v;
@@ -872,7 +874,7 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
   for (int i0 = 0; i0 < p.V; i0 += 1024) {
     if (s_base >= need) break;             // uniform: s_base is read after the barrier below
     const int i = i0 + tid;
-    const float v = i < p.V ? row[i] * p.inv_t : 0.f;
+    const float v = i < p.V ? row[i] / p.t : 0.f;
     const bool eq = i < p.V && topk_key(v) == prefix;
     const unsigned long long m = __ballot(eq);
     if (lane == 0) s_wave[wave] = (uint32_t)__popcll(m);

@@ -25,7 +25,9 @@ _workspaces: dict[Any, torch.Tensor] = {}
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    key = (device.type, device.index)
+    # one per (device, stream): calls enqueued on different streams may overlap on the GPU and the
+    # library's rule is "two calls may overlap only if they use distinct workspaces"
+    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         _workspaces.pop(key, None)
@@ -36,7 +38,7 @@ def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
 
 
 def release_workspaces() -> None:
-    """Drops the cached per-device workspaces."""
+    """Drops the cached workspaces (one per device and stream)."""
     _workspaces.clear()
 
 
@@ -57,7 +59,7 @@ class _Prepared:
     def __init__(self, hidden, lm_head, target_ids, old_logps, advantages, mask, *,
                  total_valid_token_count, epsilon_low, epsilon_high, temperature,
                  final_logit_softcap, seq_shape, chunk_tokens, sft=False, accumulate=False,
-                 entropy_coef=0.0, entropy_token_count=None, skip_masked=False):
+                 entropy_coef=0.0, entropy_token_count=None, skip_masked=False, dhidden_splits=0):
         if hidden.device.type != "cuda":
             raise RuntimeError("grpo_fused_loss needs tensors on an MI355X device (got "
                                f"{hidden.device}); there is no CPU path")
@@ -74,12 +76,8 @@ class _Prepared:
             raise ValueError(f"seq_shape {seq_shape} does not match {n} tokens")
         dev = hidden.device
         self.n, self.h, self.v, self.seq_shape, self.device = n, h, v, seq_shape, dev
-        self.hidden = hidden.to(torch.bfloat16)
-        if self.hidden.stride(1) != 1 or self.hidden.stride(0) % 8:
-            self.hidden = self.hidden.contiguous()
-        self.w = lm_head.detach().to(torch.bfloat16)
-        if self.w.stride(1) != 1 or self.w.stride(0) % 8:
-            self.w = self.w.contiguous()
+        self.hidden = self._operand(hidden.to(torch.bfloat16))
+        self.w = self._operand(lm_head.detach().to(torch.bfloat16))
         self.targets = torch.as_tensor(target_ids, device=dev).reshape(-1).to(torch.int32).contiguous()
         if self.targets.numel() != n:
             raise ValueError(f"target_ids has {self.targets.numel()} elements, expected {n}")
@@ -112,6 +110,7 @@ class _Prepared:
         d.softcap = float(final_logit_softcap or 0.0)
         d.inv_total_valid_tokens = (1.0 / tv) if tv != 0 else float("inf")
         d.grad_loss_scale = 1.0
+        d.dhidden_splits = int(dhidden_splits or 0)
         d.entropy_coef = float(entropy_coef)
         if entropy_coef != 0.0 or entropy_token_count is not None:
             cnt = float(self.mask.sum().item()) if entropy_token_count is None else float(entropy_token_count)
@@ -123,6 +122,14 @@ class _Prepared:
         self.lse = torch.empty(n, dtype=torch.float32, device=dev)
         self.ent = torch.empty(n, dtype=torch.float32, device=dev)
         self.loss = torch.empty(2, dtype=torch.float32, device=dev)   # [loss, masked-mean entropy]
+
+    @staticmethod
+    def _operand(t: torch.Tensor) -> torch.Tensor:
+        """A row-major bf16 matrix the kernels can read in place: unit column stride, row pitch a
+        multiple of 8 elements and at least the row length, 16-byte aligned base; anything else is
+        copied into a dense tensor."""
+        ok = t.stride(1) == 1 and t.stride(0) % 8 == 0 and t.stride(0) >= t.shape[1] and t.data_ptr() % 16 == 0
+        return t if ok else t.contiguous()
 
     def stream(self) -> int:
         return torch.cuda.current_stream(self.device).cuda_stream
@@ -139,7 +146,9 @@ class _Prepared:
     def forward_backward(self, d_w: Optional[torch.Tensor] = None):
         _, both = _lib.workspace_bytes(self.desc)
         ws = _workspace(self.device, both)
-        d_h = torch.empty_like(self.hidden)
+        # d_hidden is written with the row pitch of hidden (the descriptor has one ld_hidden for both)
+        ld = self.hidden.stride(0)
+        d_h = torch.empty((self.n, ld), dtype=torch.bfloat16, device=self.device)[:, : self.h]
         if d_w is None:
             d_w = torch.empty((self.h, self.w.stride(0)), dtype=torch.float32, device=self.device)
         with torch.cuda.device(self.device):
@@ -175,7 +184,7 @@ class _Prepared:
 
 _DEFAULTS = dict(total_valid_token_count=None, epsilon_low=0.2, epsilon_high=0.3, temperature=1.0,
                  final_logit_softcap=None, seq_shape=None, chunk_tokens=None, entropy_coef=0.0,
-                 entropy_token_count=None, skip_masked=False)
+                 entropy_token_count=None, skip_masked=False, dhidden_splits=0)
 
 
 def grpo_loss_value_and_grad(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
@@ -207,12 +216,13 @@ def _check_accumulator(buf: torch.Tensor, p: "_Prepared") -> None:
         raise ValueError("the lm_head gradient accumulator must be a float32 [H,V] device tensor laid out like lm_head")
 
 
-class _AccumulateTarget(threading.local):
-    buffer: Optional[torch.Tensor] = None
+class _CallMode(threading.local):
+    buffer: Optional[torch.Tensor] = None   # lm_head gradient accumulator of accumulate_lm_head_grad_into
     uses: int = 0
+    terminal: bool = False                  # inside terminal_loss()
 
 
-_accumulate_target = _AccumulateTarget()
+_accumulate_target = _CallMode()
 
 
 @contextlib.contextmanager
@@ -221,8 +231,9 @@ def accumulate_lm_head_grad_into(buffer: torch.Tensor):
     `buffer` (float32 [H,V]) inside the dW kernel and hands autograd no lm_head gradient: the
     grad-accumulation `ga + g` of plugins/training/update/train_step.py:30-33 without a
     separate [H,V] gradient tensor or a pass over it.  The loss must be terminal (it is
-    differentiated with upstream gradient 1, as training_step does); yields a counter object
-    whose `.uses` says how many calls accumulated."""
+    differentiated with upstream gradient 1, as training_step does; any other upstream gradient
+    turns buffer[0, 0] into NaN, see terminal_loss); yields a counter object whose `.uses` says
+    how many calls accumulated."""
     prev, prev_uses = _accumulate_target.buffer, _accumulate_target.uses
     _accumulate_target.buffer, _accumulate_target.uses = buffer, 0
     try:
@@ -231,10 +242,33 @@ def accumulate_lm_head_grad_into(buffer: torch.Tensor):
         _accumulate_target.buffer, _accumulate_target.uses = prev, prev_uses
 
 
+@contextlib.contextmanager
+def terminal_loss():
+    """Within this context the caller promises that every fused loss is differentiated with
+    upstream gradient exactly 1 -- what jax.value_and_grad of the reference's loss_fn does
+    (plugins/training/update/train_step.py:15-24).  The backward then hands autograd the [H,V]
+    gradient the kernel wrote as it is: no `d_w * grad` pass over 2 GB and no second copy.  The
+    promise is checked on the device without a host synchronisation: an upstream gradient other
+    than 1 adds NaN to element [0, 0] of the lm_head gradient, so a broken promise cannot go
+    unnoticed downstream."""
+    prev = _accumulate_target.terminal
+    _accumulate_target.terminal = True
+    try:
+        yield
+    finally:
+        _accumulate_target.terminal = prev
+
+
+def _poison_unless_one(grad_loss: torch.Tensor) -> torch.Tensor:
+    g = grad_loss.reshape(-1)[:1].to(torch.float32)
+    return torch.where(g == 1, torch.zeros_like(g), torch.full_like(g, float("nan")))
+
+
 class _FusedLossFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, lm_head, prepared: _Prepared, want_grad: bool):
-        ctx.direct = False
+        ctx.direct = ctx.terminal = False
+        ctx.d_w = ctx.buf = None
         if want_grad:
             buf = _accumulate_target.buffer if lm_head.requires_grad else None
             if buf is not None:
@@ -242,7 +276,11 @@ class _FusedLossFn(torch.autograd.Function):
                 prepared.desc.flags |= _lib.FLAG_DW_ACCUMULATE
                 d_h, _ = prepared.forward_backward(buf)
                 _accumulate_target.uses += 1
-                ctx.direct = True
+                ctx.direct, ctx.buf = True, buf
+                ctx.save_for_backward(d_h)
+            elif _accumulate_target.terminal:
+                d_h, d_w = prepared.forward_backward()
+                ctx.terminal, ctx.d_w = True, d_w      # kept out of save_for_backward: poisoned in place on misuse
                 ctx.save_for_backward(d_h)
             else:
                 d_h, d_w = prepared.forward_backward()
@@ -257,7 +295,13 @@ class _FusedLossFn(torch.autograd.Function):
         shape, h_dtype, w_dtype = ctx.shapes
         if ctx.direct:
             (d_h,) = ctx.saved_tensors
-            gw = None                      # already added into the accumulator by the dW kernel
+            gw = None                      # already added into the accumulator by the dW kernel ...
+            ctx.buf[0, :1].add_(_poison_unless_one(grad_loss))   # ... with upstream gradient 1
+        elif ctx.terminal:
+            (d_h,) = ctx.saved_tensors
+            d_w, ctx.d_w = ctx.d_w, None
+            d_w[0, :1].add_(_poison_unless_one(grad_loss))
+            gw = d_w if d_w.dtype == w_dtype else d_w.to(w_dtype)
         else:
             d_h, d_w = ctx.saved_tensors
             gw = (d_w * grad_loss).to(w_dtype)

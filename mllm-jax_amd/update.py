@@ -24,7 +24,7 @@ from typing import Any, Callable, Dict, Mapping, Optional
 
 import torch
 
-from .loss import accumulate_lm_head_grad_into
+from .loss import accumulate_lm_head_grad_into, terminal_loss
 
 Params = Dict[str, torch.Tensor]
 
@@ -100,15 +100,18 @@ def training_step(state: LossTrainState, inputs: Mapping[str, Any]):
     keys = [k for k, v in state.params.items() if v.requires_grad]
     direct = state.grad_accum is not None and state.lm_head_key is not None \
         and state.params[state.lm_head_key].requires_grad
+    # the loss is differentiated right here with upstream gradient 1 (value_and_grad, train_step.py:24),
+    # so the fused loss may hand autograd the kernel's [H,V] gradient as it is
     if direct:
-        with accumulate_lm_head_grad_into(state.grad_accum[state.lm_head_key]) as target:
+        with terminal_loss(), accumulate_lm_head_grad_into(state.grad_accum[state.lm_head_key]) as target:
             loss, metrics = _loss_and_aux(state, inputs)
             if target.uses != 1:
                 raise RuntimeError(f"apply_fn made {target.uses} differentiable fused-loss calls; exactly one "
                                    "may add into the lm_head accumulator per micro-step")
         keys = [k for k in keys if k != state.lm_head_key]
     else:
-        loss, metrics = _loss_and_aux(state, inputs)
+        with terminal_loss():
+            loss, metrics = _loss_and_aux(state, inputs)
     got = torch.autograd.grad(loss, [state.params[k] for k in keys], allow_unused=True) if keys else ()
     grads = {k: (g if g is not None else torch.zeros_like(state.params[k])) for k, g in zip(keys, got)}
     metrics = {k: (v.detach() if isinstance(v, torch.Tensor) else v) for k, v in metrics.items()}
@@ -138,8 +141,9 @@ def ppo_update(*, state: Any, datas: Mapping[str, Any], total_valid_token_count:
                train_step: Callable[[Any, Any], Any] = training_step,
                slice_data: Callable[[Any, int, int], Any] = slice_data,
                grad_accum_steps: int, ppo_steps: int):
-    """update/ppo.py:6-46: ppo_steps passes over the global batch in grad_accum_steps
-    micro-batches.  Every micro-batch is normalised by the GLOBAL total_valid_token_count
+    """update/ppo.py:6-46, kept statement for statement (a caller contract, not a redesign: the
+    runner and the update modules call it with exactly these keywords): ppo_steps passes over the
+    global batch in grad_accum_steps micro-batches.  Every micro-batch is normalised by the GLOBAL total_valid_token_count
     (:37); the first pass collects per_token_logps, which become old_per_token_logps for the
     later passes (:39-43).  Returns (state, datas with old_per_token_logps, last_meta, entropy)."""
     datas_dict = dict(datas)

@@ -247,10 +247,10 @@ def rms_norm(x, scale, eps=1e-6, dy=None):
 def top_k_sample(logits, k=50, t=0.9, noise=None):
     """_top_k_sampling_batched (MLLM_JAX/sample/sanple_utils.py:35-53) with the categorical draw
     written as argmax(top_logits + Gumbel noise) (what jax.random.categorical evaluates).
-    logits [B,V] float32; scaled = logits * float32(1/t) in float32; top-k in descending order,
+    logits [B,V] float32; scaled = logits / float32(t) in float32 (the reference divides, :37); top-k in descending order,
     equal values by ascending index (jax.lax.top_k); noise [B,k] or None (greedy).
     Returns (token[B], top_idx[B,k], top_val[B,k])."""
-    x = np.asarray(logits, np.float32) * np.float32(1.0 / float(t))
+    x = np.asarray(logits, np.float32) / np.float32(t)
     b, v = x.shape
     order = np.lexsort((np.broadcast_to(np.arange(v), x.shape), -x.astype(np.float64)), axis=-1)[:, :k]
     top_val = np.take_along_axis(x, order, axis=-1)

@@ -141,6 +141,24 @@ def test_config3_full_size_runs_and_is_consistent():
     assert not dh[wl["mask"] == 0].any() and dh[wl["mask"] > 0].float().abs().sum() > 0
     rs = dw.double().sum(-1).abs().max().item()
     assert rs <= 1e-3 * dw.double().abs().sum(-1).max().item()
+    # all 32768 tokens against the oracle, in two halves of rows (the second half is the chunk the
+    # kernels reach with a non-zero chunk origin and an accumulating dW); the halves' d_lm_head
+    # shares add up to the whole gradient
+    n = wl["hidden"].shape[0]
+    ref_dw = None
+    for half in (torch.arange(0, n // 2), torch.arange(n // 2, n)):
+        ref = O.grpo_loss_chunked_torch(
+            wl["hidden"], wl["lm_head"], wl["target_ids"], wl["old_logps"], wl["advantages"], wl["mask"],
+            total_valid_token_count=wl["total_valid_token_count"], epsilon_low=cfg.eps_low,
+            epsilon_high=cfg.eps_high, final_logit_softcap=cfg.softcap, chunk=1024, rows=half, device="cuda:0",
+            as_numpy=False)
+        rows = half.to(dh.device)
+        _check_against(ref, met, dh, dw, rows=rows)
+        assert _rel(dh[rows].float(), ref["d_hidden"][rows]) <= GRAD_RTOL
+        ref_dw = ref["d_lm_head"] if ref_dw is None else ref_dw.add_(ref["d_lm_head"])
+        del ref
+    assert _rel(dw, ref_dw) <= GRAD_RTOL
+    del ref_dw
     M.release_workspaces()
     torch.cuda.empty_cache()
 

@@ -1,0 +1,80 @@
+"""GPU: the terminal-loss path of the autograd function.  Inside terminal_loss() the backward hands
+autograd the [H,V] gradient tensor the kernel wrote (no multiply, no copy); a broken promise
+(upstream gradient != 1) shows up as NaN in element [0,0] of the lm_head gradient."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import grpo_oracle as O
+from test_gpu_parity import GRAD_RTOL, _case, _rel
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(seed):
+    hid, w, y, adv, mask = _case(seed, 256, 64, 1000, 2)
+    ref = O.grpo_loss(hid.float().numpy(), w.float().numpy(), y.numpy(), None, adv.numpy(), mask.numpy())
+    dev = torch.device("cuda:0")
+    hp = hid.to(dev).requires_grad_()
+    wp = w.float().to(dev).requires_grad_()          # float32 master weights, as in the reference
+    args = (y.to(dev), None, adv.to(dev), mask.to(dev))
+    return ref, hp, wp, args
+
+
+def test_terminal_backward_returns_the_kernel_output_itself():
+    import mllm_jax_amd as M
+    from mllm_jax_amd import loss as L
+    ref, hp, wp, args = _setup(51)
+    seen = {}
+    orig = L._Prepared.forward_backward
+
+    def spy(self, d_w=None):
+        d_h, d_wv = orig(self, d_w)
+        seen["ptr"] = d_wv.data_ptr()
+        return d_h, d_wv
+
+    L._Prepared.forward_backward = spy
+    try:
+        with M.terminal_loss():
+            out = M.grpo_fused_loss(hp, wp, *args)
+            out["loss"].backward()
+    finally:
+        L._Prepared.forward_backward = orig
+    torch.cuda.synchronize()
+    assert wp.grad.data_ptr() == seen["ptr"], "the [H,V] gradient was copied or rescaled on the way to autograd"
+    assert _rel(wp.grad.cpu().numpy(), ref["d_lm_head"]) <= GRAD_RTOL
+    assert _rel(hp.grad.float().cpu().numpy(), ref["d_hidden"]) <= GRAD_RTOL
+
+
+def test_broken_promise_poisons_the_lm_head_gradient():
+    import mllm_jax_amd as M
+    ref, hp, wp, args = _setup(52)
+    with M.terminal_loss():
+        out = M.grpo_fused_loss(hp, wp, *args)
+        (out["loss"] * 0.5).backward()
+    torch.cuda.synchronize()
+    assert torch.isnan(wp.grad[0, 0]) and torch.isfinite(wp.grad[0, 1:]).all() and torch.isfinite(wp.grad[1:]).all()
+    # outside the context the general path scales correctly
+    hp.grad = None
+    wp.grad = None
+    out = M.grpo_fused_loss(hp, wp, *args)
+    (out["loss"] * 0.5).backward()
+    torch.cuda.synchronize()
+    assert _rel(wp.grad.cpu().numpy(), 0.5 * ref["d_lm_head"]) <= GRAD_RTOL
+
+
+def test_accumulating_with_a_scaled_loss_poisons_the_accumulator():
+    import mllm_jax_amd as M
+    ref, hp, wp, args = _setup(53)
+    acc = torch.zeros_like(wp)
+    with M.accumulate_lm_head_grad_into(acc):
+        out = M.grpo_fused_loss(hp, wp, *args)
+        (out["loss"] / 2).backward()
+    torch.cuda.synchronize()
+    assert torch.isnan(acc[0, 0]) and torch.isfinite(acc[0, 1:]).all()
+    acc.zero_()
+    with M.accumulate_lm_head_grad_into(acc):
+        out = M.grpo_fused_loss(hp, wp, *args)
+        out["loss"].backward()
+    torch.cuda.synchronize()
+    assert _rel(acc.cpu().numpy(), ref["d_lm_head"]) <= GRAD_RTOL

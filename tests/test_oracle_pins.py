@@ -418,3 +418,37 @@ def test_gae_by_hand_with_discount_and_values():
     d2 = 2.0 - (-0.1); d1 = g * (-0.1) - 0.2
     np.testing.assert_allclose(adv, [[0.0, d1 + g * lam * d2, d2, 0.0]], atol=1e-6)
     np.testing.assert_allclose(ret, adv + v, atol=1e-7)
+
+
+def test_lm_head_logits_against_brute_force_and_tanh_identity(rng):
+    """lm_head_logits is hidden @ lm_head with the [in, out] kernel layout (a transposed operand or a
+    [V,H] layout fails the brute-force sum), and the softcap is cap*tanh(z/cap): odd, bounded by the
+    cap, the identity for |z| << cap."""
+    hid = rng.standard_normal((5, 7))
+    w = rng.standard_normal((7, 11))
+    z = O.lm_head_logits(hid, w)
+    brute = np.array([[sum(hid[t, k] * w[k, v] for k in range(7)) for v in range(11)] for t in range(5)])
+    np.testing.assert_allclose(z, brute, atol=1e-12)
+    np.testing.assert_allclose(z, torch.from_numpy(hid) @ torch.from_numpy(w), atol=1e-12)
+    zc = O.lm_head_logits(hid * 20, w, softcap=30.0)
+    raw = O.lm_head_logits(hid * 20, w)
+    assert np.abs(zc).max() < 30.0 and np.abs(raw).max() > 30.0
+    np.testing.assert_allclose(zc, -O.lm_head_logits(-hid * 20, w, softcap=30.0), atol=1e-12)
+    np.testing.assert_allclose(O.lm_head_logits(hid * 1e-3, w, softcap=30.0), raw * (1e-3 / 20), rtol=1e-6)
+    # inverse: atanh(zc/cap)*cap recovers the raw logits
+    np.testing.assert_allclose(np.arctanh(zc / 30.0) * 30.0, raw, rtol=1e-9)
+
+
+def test_top_k_divides_by_temperature_like_the_reference():
+    """sanple_utils.py:37 computes logits / t.  In float32 that differs from logits * (1/t) by an ulp
+    for some values, which can reorder near-ties; the oracle must divide."""
+    x = np.array([[1.0000001, 1.0, 3.3, 0.7, 2.9000001, 2.9]], np.float32)
+    t = np.float32(0.9)
+    _, idx, val = O.top_k_sample(x, k=6, t=float(t), noise=None)
+    np.testing.assert_array_equal(val[0], np.sort((x / t)[0])[::-1])
+    assert val.dtype == np.float32
+    # a value where the two formulations differ in the last bit
+    xs = np.arange(1, 4097, dtype=np.float32) / np.float32(7.0)
+    assert np.any(xs / t != xs * np.float32(1.0 / float(t)))
+    _, _, v2 = O.top_k_sample(xs[None, :], k=8, t=float(t), noise=None)
+    np.testing.assert_array_equal(v2[0], np.sort(xs / t)[::-1][:8])
