@@ -63,34 +63,42 @@ def _vendor_gemm(torch, hidden, w, mask, n, h, v, reps=5):
 
 
 class _SmiSampler:
-    """Polls `rocm-smi -P -c -t --json` in a thread while the timed loop runs (power, shader clock and
-    temperature as the driver reports them); the GPU work is not touched."""
+    """Polls `amd-smi metric -p -c -t --json` in a thread while the timed loop runs (socket power, the
+    shader clock of every XCD and the hotspot temperature as the driver reports them); the GPU work is
+    not touched."""
 
-    def __init__(self, period_s=0.2):
+    def __init__(self, period_s=0.15):
         import threading
         self.period, self.samples, self._stop = period_s, [], threading.Event()
         self._thread = threading.Thread(target=self._run, daemon=True)
 
+    @staticmethod
+    def _num(x):
+        if isinstance(x, dict):
+            x = x.get("value")
+        return float(x) if isinstance(x, (int, float)) else None
+
     def _run(self):
-        import re
         import subprocess
         while not self._stop.is_set():
             try:
-                out = subprocess.run(["rocm-smi", "-P", "-c", "-t", "--json"], capture_output=True, text=True,
-                                     timeout=10).stdout
-                card = next(iter(json.loads(out).values()))
+                out = subprocess.run(["amd-smi", "metric", "-p", "-c", "-t", "--json"], capture_output=True,
+                                     text=True, timeout=10).stdout
+                doc = json.loads(out)
+                gpu = (doc.get("gpu_data") if isinstance(doc, dict) else doc)[0]
                 rec = {}
-                for k, v in card.items():
-                    m = re.search(r"[-+]?\d+(\.\d+)?", str(v))
-                    if not m:
-                        continue
-                    kl = k.lower()
-                    if "power" in kl and "max" not in kl:
-                        rec["power_w"] = float(m.group())
-                    elif kl.startswith("sclk"):
-                        rec["sclk_mhz"] = float(m.group())
-                    elif "junction" in kl:
-                        rec["junction_c"] = float(m.group())
+                pw = self._num(gpu.get("power", {}).get("socket_power"))
+                if pw is not None:
+                    rec["power_w"] = pw
+                clks = [self._num(v.get("clk")) for k, v in gpu.get("clock", {}).items()
+                        if k.startswith("gfx_") and isinstance(v, dict)]
+                clks = [c for c in clks if c is not None]
+                if clks:
+                    rec["sclk_mhz"] = round(sum(clks) / len(clks), 1)
+                temp = gpu.get("temperature", {})
+                hot = self._num(temp.get("hotspot")) if isinstance(temp, dict) else None
+                if hot is not None:
+                    rec["junction_c"] = hot
                 if rec:
                     rec["t"] = round(time.perf_counter(), 3)
                     self.samples.append(rec)

@@ -163,7 +163,9 @@ enum {
   MJ_GRPO_K_DHIDDEN_REDUCE = 4,
   MJ_GRPO_K_DW = 5,
   MJ_GRPO_K_REDUCE_LOSS = 6,
-  MJ_GRPO_K_COUNT = 7
+  MJ_GRPO_K_SCALE_HIDDEN = 7,
+  MJ_GRPO_K_RESCUE = 8,       /* the three launches of the running-maximum rescue pass together */
+  MJ_GRPO_K_COUNT = 9
 };
 int mj_grpo_profile_begin(int max_launches);
 int mj_grpo_profile_end(double* total_ms /* [MJ_GRPO_K_COUNT] */, int* launches /* [MJ_GRPO_K_COUNT] */);

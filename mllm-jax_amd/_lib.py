@@ -20,7 +20,7 @@ EXPORTS = ("mj_grpo_version", "mj_grpo_last_error", "mj_grpo_workspace_bytes", "
            "mj_grpo_group_advantages", "mj_grpo_advantages", "mj_grpo_gae", "mj_rmsnorm_forward", "mj_sample_logits", "mj_sample_top_k", "mj_rmsnorm_workspace_bytes", "mj_rmsnorm_backward")
 
 KERNEL_NAMES = ("k_logits_stats", "k_finalize", "k_dz", "k_dhidden", "k_dhidden_reduce", "k_dw",
-                "k_reduce_loss")
+                "k_reduce_loss", "k_scale_hidden", "k_rescue")
 
 
 class MjGrpoDesc(C.Structure):

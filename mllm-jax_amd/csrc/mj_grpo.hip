@@ -53,6 +53,7 @@ struct Timed {
 
 constexpr int BM = 256, BN = 256;          // tile of all three contractions
 constexpr int64_t kDefaultChunk = 16384;   // tokens whose logits live in the workspace at once
+constexpr int kRescueGrid = 256;           // workgroups of the rescue pass (one per CU)
 
 inline int64_t rup(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
 
@@ -61,7 +62,7 @@ struct Plan {
   int dh_splits;          // vocab splits of the dHidden product (1 = none)
   int64_t dh_k_per_split;
   // byte offsets into the workspace
-  size_t zy, term, eterm, pm, pl, ps, plt, g, ge, hent, zt, part, total_fwd, total_bwd;
+  size_t zy, term, eterm, pm, pl, ps, plt, g, ge, hent, state, rs, hs, zt, part, total_fwd, total_bwd;
   // token compaction (MJ_GRPO_FLAG_SKIP_MASKED): slot-order copies of the inputs and outputs
   bool compact;
   size_t perm, n_live, hid_p, tgt_p, fin_p[5], fout_p[3], dh_p;
@@ -111,7 +112,7 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   if (chunk > p->N) chunk = p->N;
   p->chunk = chunk;
   p->n_pad = rup(chunk, 256);
-  p->ld_z = p->n_pad;
+  p->ld_z = p->V;               // rows of the 16-bit matrix: V % 8 == 0 keeps them 16-byte aligned
   p->parts = 2 * ((p->V + BM - 1) / BM);
   if (d->dhidden_splits > 32) return fail(MJ_GRPO_ERR_SHAPE, "dhidden_splits must be <= 32 (got %u)", d->dhidden_splits);
   p->dh_splits = d->dhidden_splits ? (int)d->dhidden_splits : pick_splits((p->n_pad / BM) * ((p->H + BN - 1) / BN));
@@ -128,6 +129,7 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   p->g = take((size_t)p->n_pad * 4);
   p->ge = take((size_t)p->n_pad * 4);
   p->hent = take((size_t)p->n_pad * 4);
+  p->state = take(256);
   p->compact = (d->flags & MJ_GRPO_FLAG_SKIP_MASKED) != 0;
   if (p->compact) {
     p->perm = take((size_t)p->N * 4);
@@ -139,7 +141,9 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   }
   p->total_fwd = o;
   p->dh_p = take(p->compact ? (size_t)p->N * p->H * 2 : 0);
-  p->zt = take((size_t)p->V * p->ld_z * 2);
+  p->rs = take((size_t)p->n_pad * 4);
+  p->hs = take((size_t)p->n_pad * p->H * 2);
+  p->zt = take((size_t)p->n_pad * p->ld_z * 2);
   p->part = take(p->dh_splits > 1 ? (size_t)p->dh_splits * p->n_pad * p->H * 4 : 0);
   p->total_bwd = o;
   return MJ_GRPO_OK;
@@ -215,7 +219,20 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
   const float gscale = d->grad_loss_scale;
   const size_t lds = mj::GemmTN<BM, BN>::kLdsBytes;
 
-  if ((rc = enable_lds(mj::k_logits_stats<BM, BN>))) return rc;
+  // Which statistics the logits epilogue keeps (mj::StatsMode): sums of exp(z) without a running
+  // maximum plus E = exp(z) for the backward -- with a kStatsMax rescue pass enqueued behind it that
+  // leaves at once unless the range check failed -- or, where that form does not apply, kStatsMax.
+  const bool exp_mode = mode != kBackwardOnly && d->temperature == 1.0f && d->entropy_coef == 0.f;
+  int* state = (int*)(ws + p.state);
+  float* rs = (float*)(ws + p.rs);
+  uint16_t* hs = (uint16_t*)(ws + p.hs);
+  if (mode == kBackwardOnly) {
+    if ((rc = enable_lds(mj::k_logits_stats<BM, BN, mj::kStatsGrad, false>))) return rc;
+  } else {
+    if (exp_mode && (rc = enable_lds(mj::k_logits_stats<BM, BN, mj::kStatsExp, false>))) return rc;
+    if (exp_mode && (rc = enable_lds(mj::k_logits_stats<BM, BN, mj::kStatsMax, true>))) return rc;
+    if (!exp_mode && (rc = enable_lds(mj::k_logits_stats<BM, BN, mj::kStatsMax, false>))) return rc;
+  }
   if (bwd) {
     if ((rc = enable_lds(mj::k_dhidden<BM, BN>))) return rc;
     if ((rc = enable_lds(mj::k_dw<BM, BN>))) return rc;
@@ -259,48 +276,87 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     const int nc = (int)((p.N - c0 < p.chunk) ? p.N - c0 : p.chunk);
     const int n_pad = (int)rup(nc, 256);
     const __bf16* hid_c = (const __bf16*)hidden + c0 * ld_hid;
-    {
-      mj::LogitsArgs a;
-      a.w = (const __bf16*)lm_head; a.hid = hid_c; a.ld_w = d->ld_w; a.ld_hid = ld_hid;
-      a.V = V; a.n = nc; a.H = H; a.cap = d->softcap;
-      a.zt = bwd ? zt : nullptr; a.ld_z = p.ld_z;
-      a.pm = pm; a.pl = pl; a.ps = ps; a.plt = plt; a.inv_t = inv_t; a.ld_p = p.n_pad;
-      a.targets = targets + c0; a.zy = zy + c0; a.n_live = n_live; a.c0 = (int)c0;
-      const mj::TileMap map((V + BM - 1) / BM, (nc + BN - 1) / BN, 1);
-      Timed t(MJ_GRPO_K_LOGITS_STATS, st);
-      mj::k_logits_stats<BM, BN><<<map.items(), mj::kThreads, lds, st>>>(a, map);
-    }
-    if (mode != kBackwardOnly) {
-      mj::FinalizeArgs f;
-      f.pm = pm; f.pl = pl; f.ps = ps; f.plt = plt; f.inv_t = inv_t; f.ld_p = p.n_pad; f.parts = (int)p.parts;
-      f.n = nc; f.n_pad = n_pad; f.zy = zy + c0;
-      f.old_logp = old_logp ? old_logp + c0 : nullptr;
-      f.adv = adv ? adv + c0 : nullptr; f.mask = mask + c0;
-      f.eps_low = d->eps_low; f.eps_high = d->eps_high; f.inv_tv = d->inv_total_valid_tokens;
-      f.gscale = gscale; f.sft = sft ? 1 : 0;
-      f.logp = logp + c0; f.lse = lse + c0; f.ent = ent ? ent + c0 : nullptr;
-      f.term = term + c0; f.g = bwd ? g : nullptr;
-      f.ent_coef = d->entropy_coef; f.inv_ent_cnt = d->inv_entropy_count; f.eterm = eterm + c0;
-      f.ge = bonus ? ge : nullptr; f.hent = bonus ? hent : nullptr;
+    mj::LogitsArgs a;
+    a.w = (const __bf16*)lm_head; a.hid = hid_c; a.ld_w = d->ld_w; a.ld_hid = ld_hid;
+    a.V = V; a.n = nc; a.H = H; a.cap = d->softcap;
+    a.zt = bwd ? zt : nullptr; a.ld_z = p.ld_z;
+    a.pm = pm; a.pl = pl; a.ps = ps; a.plt = plt; a.inv_t = inv_t; a.ld_p = p.n_pad;
+    a.targets = targets + c0; a.zy = zy + c0; a.n_live = n_live; a.c0 = (int)c0;
+    a.mask = mask + c0; a.lse = nullptr; a.g = g; a.state = state;
+    const mj::TileMap map((V + BM - 1) / BM, (nc + BN - 1) / BN, 1);
+
+    mj::FinalizeArgs f;
+    f.pm = pm; f.pl = pl; f.ps = ps; f.plt = plt; f.inv_t = inv_t; f.ld_p = p.n_pad; f.parts = (int)p.parts;
+    f.n = nc; f.n_pad = n_pad; f.zy = zy + c0;
+    f.old_logp = old_logp ? old_logp + c0 : nullptr;
+    f.adv = adv ? adv + c0 : nullptr; f.mask = mask + c0;
+    f.eps_low = d->eps_low; f.eps_high = d->eps_high; f.inv_tv = d->inv_total_valid_tokens;
+    f.gscale = gscale; f.sft = sft ? 1 : 0;
+    f.logp = logp ? logp + c0 : nullptr; f.lse = lse ? lse + c0 : nullptr; f.ent = ent ? ent + c0 : nullptr;
+    f.term = term + c0; f.g = bwd ? g : nullptr;
+    f.ent_coef = d->entropy_coef; f.inv_ent_cnt = d->inv_entropy_count; f.eterm = eterm + c0;
+    f.ge = bonus ? ge : nullptr; f.hent = bonus ? hent : nullptr;
+    f.rs = bwd ? rs : nullptr; f.zt = zt; f.ld_z = p.ld_z; f.targets = targets + c0; f.V = V; f.cap = d->softcap;
+    f.state = state; f.rescue = 0;
+
+    mj::DzArgs z;
+    z.zt = zt; z.ld_z = p.ld_z;
+    z.lse = (mode == kBackwardOnly ? saved_lse : lse) + c0; z.g = g; z.targets = targets + c0;
+    z.ge = bonus ? ge : nullptr; z.hent = bonus ? hent : nullptr;
+    z.V = V; z.n = nc; z.cap = d->softcap; z.n_live = n_live; z.c0 = (int)c0; z.state = state; z.rescue = 0;
+    const unsigned dz_grid = (unsigned)(nc < 8192 ? nc : 8192);
+
+    if (mode == kBackwardOnly) {
+      {
+        Timed t(MJ_GRPO_K_FINALIZE, st);
+        mj::k_coeff_from_saved<<<(n_pad + 255) / 256, 256, 0, st>>>(
+            saved_logp + c0, old_logp ? old_logp + c0 : nullptr, adv ? adv + c0 : nullptr, mask + c0, nc, n_pad,
+            d->eps_low, d->eps_high, d->inv_total_valid_tokens, gscale * inv_t, sft ? 1 : 0, g);
+      }
+      a.lse = saved_lse + c0;
+      {
+        Timed t(MJ_GRPO_K_LOGITS_STATS, st);
+        mj::k_logits_stats<BM, BN, mj::kStatsGrad, false><<<map.items(), mj::kThreads, lds, st>>>(a, map);
+      }
       Timed t(MJ_GRPO_K_FINALIZE, st);
-      mj::k_finalize<<<n_pad / 64, 64 * mj::kFinSlices, 0, st>>>(f);
+      mj::k_patch_grad<<<(nc + 255) / 256, 256, 0, st>>>(zt, p.ld_z, zy + c0, saved_lse + c0, g, targets + c0, nc, V,
+                                                         d->softcap, state);
+    } else if (exp_mode) {
+      {
+        Timed t(MJ_GRPO_K_LOGITS_STATS, st);
+        mj::k_logits_stats<BM, BN, mj::kStatsExp, false><<<map.items(), mj::kThreads, lds, st>>>(a, map);
+      }
+      {
+        Timed t(MJ_GRPO_K_FINALIZE, st);
+        mj::k_finalize<mj::kStatsExp><<<n_pad / 64, 64 * mj::kFinSlices, 0, st>>>(f);
+      }
+      if (bwd) {
+        const int64_t work = (int64_t)nc * (H / 8);
+        Timed t(MJ_GRPO_K_SCALE_HIDDEN, st);
+        mj::k_scale_hidden<<<(unsigned)((work + 255) / 256), 256, 0, st>>>((const uint16_t*)hid_c, ld_hid, rs, nc, H, hs);
+      }
+      // the rescue: the same chunk with a running maximum; every workgroup leaves at once unless the
+      // range check in k_finalize failed
+      Timed t(MJ_GRPO_K_RESCUE, st);
+      f.rescue = 1; z.rescue = 1;
+      mj::k_logits_stats<BM, BN, mj::kStatsMax, true><<<kRescueGrid, mj::kThreads, lds, st>>>(a, map);
+      mj::k_finalize<mj::kStatsMax><<<n_pad / 64, 64 * mj::kFinSlices, 0, st>>>(f);
+      if (bwd) mj::k_dz<<<dz_grid, 256, 0, st>>>(z);
     } else {
-      Timed t(MJ_GRPO_K_FINALIZE, st);
-      mj::k_coeff_from_saved<<<(n_pad + 255) / 256, 256, 0, st>>>(
-          saved_logp + c0, old_logp ? old_logp + c0 : nullptr, adv ? adv + c0 : nullptr, mask + c0, nc, n_pad,
-          d->eps_low, d->eps_high, d->inv_total_valid_tokens, gscale * inv_t, sft ? 1 : 0, g);
+      {
+        Timed t(MJ_GRPO_K_LOGITS_STATS, st);
+        mj::k_logits_stats<BM, BN, mj::kStatsMax, false><<<map.items(), mj::kThreads, lds, st>>>(a, map);
+      }
+      {
+        Timed t(MJ_GRPO_K_FINALIZE, st);
+        mj::k_finalize<mj::kStatsMax><<<n_pad / 64, 64 * mj::kFinSlices, 0, st>>>(f);
+      }
+      if (bwd) {
+        Timed t(MJ_GRPO_K_DZ, st);
+        mj::k_dz<<<dz_grid, 256, 0, st>>>(z);
+      }
     }
     if (bwd) {
-      mj::DzArgs z;
-      z.zt = zt; z.ld_z = p.ld_z;
-      z.lse = (mode == kBackwardOnly ? saved_lse : lse) + c0; z.g = g; z.targets = targets + c0;
-      z.ge = bonus ? ge : nullptr; z.hent = bonus ? hent : nullptr;
-      z.V = V; z.n = nc; z.n_pad = n_pad; z.cap = d->softcap; z.n_live = n_live; z.c0 = (int)c0;
-      {
-        Timed t(MJ_GRPO_K_DZ, st);
-        mj::k_dz<<<dim3((V + mj::kDzRows - 1) / mj::kDzRows, n_pad / 256), 256, 0, st>>>(z);
-      }
-
       // the split count was planned for a full chunk; a shorter last chunk keeps it (the partial
       // buffer is sized for it) unless it has a single split anyway
       mj::DhArgs h;
@@ -308,7 +364,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       h.n = nc; h.n_pad = n_pad; h.H = H; h.V = V;
       h.splits = p.dh_splits; h.k_per_split = (int)p.dh_k_per_split;
       h.dh = (uint16_t*)d_hidden + c0 * ld_dh; h.ld_dh = ld_dh;
-      h.part = part; h.n_live = n_live; h.c0 = (int)c0;
+      h.part = part; h.n_live = n_live; h.c0 = (int)c0; h.rs = rs; h.state = state;
       const mj::TileMap mh((nc + BM - 1) / BM, (H + BN - 1) / BN, 0, 2, h.splits);
       {
         Timed t(MJ_GRPO_K_DHIDDEN, st);
@@ -318,13 +374,13 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
         const int64_t work = (int64_t)nc * (H / 4);
         Timed t(MJ_GRPO_K_DHIDDEN_REDUCE, st);
         mj::k_dhidden_reduce<<<(unsigned)((work + 255) / 256), 256, 0, st>>>(part, h.splits, nc, n_pad, H, h.dh,
-                                                                           h.ld_dh);
+                                                                           h.ld_dh, rs, state);
       }
 
       mj::DwArgs w;
-      w.dzt = (const __bf16*)zt; w.hid = hid_c; w.ld_z = p.ld_z; w.ld_hid = ld_hid;
+      w.dzt = (const __bf16*)zt; w.hid = hid_c; w.hs = (const __bf16*)hs; w.ld_z = p.ld_z; w.ld_hid = ld_hid;
       w.H = H; w.V = V; w.n = nc;
-      w.dw = d_w; w.ld_dw = d->ld_w; w.n_live = n_live; w.c0 = (int)c0;
+      w.dw = d_w; w.ld_dw = d->ld_w; w.n_live = n_live; w.c0 = (int)c0; w.state = state;
       w.accumulate = (c0 > 0 || (d->flags & MJ_GRPO_FLAG_DW_ACCUMULATE)) ? 1 : 0;
       const mj::TileMap mw((V + BM - 1) / BM, (H + BN - 1) / BN, 0);
       {
@@ -603,7 +659,10 @@ int mj_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x, int64_t ld
 }  // extern "C"
 
 // Explicit instantiations of the tile kernels used above.
-template __global__ void mj::k_logits_stats<256, 256>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsExp, false>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsMax, false>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsMax, true>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsGrad, false>(mj::LogitsArgs, mj::TileMap);
 template __global__ void mj::k_dhidden<256, 256>(mj::DhArgs, mj::TileMap);
 template __global__ void mj::k_dw<256, 256>(mj::DwArgs, mj::TileMap);
 template __global__ void mj::k_logits_rows<256, 256>(mj::LogitsRowsArgs, mj::TileMap);

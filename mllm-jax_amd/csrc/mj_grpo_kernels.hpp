@@ -2,16 +2,17 @@
 //
 // Per token chunk of n rows (n <= chunk_tokens):
 //   k_logits_stats  : logits^T tile [vocab x tokens] = W^T * hidden^T on MFMA, W and hidden read in
-//                     place; the epilogue applies the softcap, reduces (max, sum exp, sum exp*z)
-//                     per token over the tile's vocab rows, picks out the sampled token's logit
-//                     and (training) stores the capped logits as IEEE half, transposed [V, n].
-//   k_finalize      : merges the per-tile statistics -> lse, logp, entropy, ratio / clip / min
-//                     surrogate, per-token loss term and dloss/dlogp.
-//   k_dz            : in place, logits^T -> dZ^T = g * (onehot - exp(z - lse)) * softcap' (bf16).
-//   k_dhidden       : dHidden[n,H] = dZ * W^T  (dZ read k-major from dZ^T), optionally split over
-//                     the vocab into fp32 partial sums that k_dhidden_reduce adds up.
-//   k_dw            : dW^T tile [vocab x hidden] = dZ^T * hidden, written / accumulated into
-//                     dW[H,V] with 16-byte accesses.
+//                     place; the epilogue applies the softcap, reduces (sum exp, sum exp*z) per token
+//                     over the tile's vocab rows, picks out the sampled token's logit and (training)
+//                     stores a 16-bit row-major [n, V] matrix for the backward (see StatsMode).
+//   k_finalize      : adds up the per-tile statistics -> lse, logp, entropy, ratio / clip / min
+//                     surrogate, per-token loss term, dloss/dlogp, the row scale of E and its
+//                     one-hot patch.
+//   k_dhidden       : dHidden[n,H] = rowscale * (E or dZ) * W^T, optionally split over the vocab into
+//                     fp32 partial sums that k_dhidden_reduce adds up.
+//   k_dw            : dW^T tile [vocab x hidden] = (E or dZ)^T * (rs * hidden or hidden), written /
+//                     accumulated into dW[H,V] with 16-byte accesses.
+//   k_dz            : only behind a kStatsMax pass: in place, logits -> dZ (bf16).
 // Nothing here allocates; all buffers come from the caller's workspace.
 #pragma once
 #include "gemm_tn.hpp"
@@ -74,13 +75,32 @@ MJ_DEV int live_pad(const int* n_live, int c0, int n_pad) {
 }
 
 // ----------------------------------------------------------------------------- logits + stats
+// What the epilogue of the logits product keeps for a chunk of tokens:
+//   kStatsExp  : per (vocab half-tile, token) the sums of e = exp(z) and e * z with NO running
+//                maximum (valid while logsumexp(z) stays within +-60, which k_finalize checks for
+//                every token) and, when a backward follows, the row-major 16-bit matrix
+//                E[t, v] = bf16(exp(z) * cap'(z)) with zero rows for masked tokens.  Since
+//                dZ[t, v] = rs_t * (E[t, v] - onehot patch) with rs_t = -g_t / sum_v exp(z), the two
+//                backward products read E as it is: k_dhidden scales its output rows by rs_t, k_dw
+//                reads rs_t * hidden, and no pass over [n, V] is needed to form dZ.
+//   kStatsMax  : the same sums relative to the per-tile maximum (any logit range) and the capped
+//                logits as IEEE half; k_dz turns those into dZ in place.  Used with temperature != 1,
+//                with the entropy bonus, and as the rescue when kStatsExp's range check fails.
+//   kStatsGrad : backward from a saved forward: lse and dloss/dlogp are inputs, so the epilogue writes
+//                dZ = -g * p * cap' directly (k_patch_grad adds the one-hot term).
+// state[0] tells the backward products what the 16-bit matrix holds: 0 = E (scale by rs, read
+// rs * hidden), 1 = dZ itself.
+enum StatsMode { kStatsExp = 0, kStatsMax = 1, kStatsGrad = 2 };
+
+constexpr float kExpSumMin = 0x1p-86f, kExpSumMax = 0x1p86f;   // logsumexp within about +-59.6
+
 struct LogitsArgs {
   const __bf16* w;       // lm_head [H, ld_w]
   const __bf16* hid;     // chunk origin, [n, ld_hid]
   int64_t ld_w, ld_hid;
   int V, n, H;
   float cap;             // 0 = off
-  uint16_t* zt;          // [V, ld_z] half logits^T of the chunk, or nullptr (forward only)
+  uint16_t* zt;          // [n, ld_z] 16-bit rows of the chunk (see StatsMode), or nullptr (forward only)
   int64_t ld_z;
   float *pm, *pl, *ps;   // per (vocab half-tile, token) partial max / sum e / sum e*z, ld = ld_p
   float* plt;            // temperature != 1 only: sum e^((z-max)/T), and ps then holds sum e^((z-max)/T)*z
@@ -90,14 +110,46 @@ struct LogitsArgs {
   float* zy;                // chunk origin: capped logit of the sampled token
   const int* n_live;        // null, or device count of leading tokens (from token c0 on) that need a backward
   int c0;
+  const float* mask;        // kStatsExp: chunk origin; tokens with mask == 0 get zero rows of E
+  const float *lse, *g;     // kStatsGrad: chunk-local saved logsumexp [n] and dloss/dlogp [n_pad]
+  int* state;
 };
 
-template <int BM, int BN>
-__global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap map) {
+MJ_DEV uint32_t pack_bf16(float a, float b) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
+MJ_DEV uint32_t pack_f16(float a, float b) {   // clamped to the finite half range, round to nearest even
+  typedef __attribute__((ext_vector_type(2))) float f32x2;
+  typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+  const f32x2 v = {__builtin_amdgcn_fmed3f(a, -65504.f, 65504.f), __builtin_amdgcn_fmed3f(b, -65504.f, 65504.f)};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+
+// Eight values of one token: a lane's rows 0..3 of two consecutive 8-row groups of the MFMA layout.
+// The lanes l and l + 32 hold rows 4..7 of the same groups for the same token; after exchanging
+// one half with the partner each lane owns eight CONSECUTIVE vocab entries and stores them with
+// one 16-byte access (`voff` carries the lane's 16 bytes of the 32).
+template <bool HALF>
+MJ_DEV void store_rows8(const float (&v)[8], uint32_t keep, __amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff) {
+  uint32_t a0, a1, b0, b1;
+  if (HALF) {
+    a0 = pack_f16(v[0], v[1]); a1 = pack_f16(v[2], v[3]); b0 = pack_f16(v[4], v[5]); b1 = pack_f16(v[6], v[7]);
+  } else {
+    a0 = pack_bf16(v[0], v[1]); a1 = pack_bf16(v[2], v[3]); b0 = pack_bf16(v[4], v[5]); b1 = pack_bf16(v[6], v[7]);
+  }
+  // v_permlane32_swap: the first operand of lanes 32..63 <-> the second operand of lanes 0..31
+  const auto s0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
+  const auto s1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
+  const u32x4 out = {s0[0] & keep, s1[0] & keep, s0[1] & keep, s1[1] & keep};
+  __builtin_amdgcn_raw_buffer_store_b128(out, rs, voff, soff, 0);
+}
+
+// One 256 x 256 tile: logits^T [vocab x tokens] = W^T * hidden^T on MFMA, then the epilogue of MODE.
+template <int BM, int BN, int MODE>
+MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
   using G = GemmTN<BM, BN, kKRow, kRowK>;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  int tm, tn, split;
-  if (!map.tile(blockIdx.x, tm, tn, split)) return;
   const int m0 = tm * BM, n0 = tn * BN;
   G g;
   g.run(p.w + m0, p.V - m0, p.ld_w, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0, p.ld_hid, p.H, smem);
@@ -107,16 +159,19 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
   const int vwave = m0 + wm * G::WM;             // first vocab row of this wavefront
   const int vbase = vwave + lhi * 4;             // + mi*32 + (r/4)*8 + r%4
+  const int t0 = n0 + wn * G::WN;                // first token of this wavefront
   const bool tail = (m0 + BM > p.V);
   const float inv_cap = p.cap > 0.f ? 1.f / p.cap : 0.f;
+  const float inv_cap2 = inv_cap * inv_cap;
   const int zt_cols = live_pad(p.n_live, p.c0, (p.n + 255) & ~255);
-  // this wavefront's 128 rows of logits^T; rows at or past V fall outside and are dropped
+  // this wavefront's 128 token rows of the 16-bit matrix; rows at or past n fall outside and are dropped
   const uint32_t ldz2 = (uint32_t)p.ld_z * 2;
-  const int zrows = min(max(p.V - vwave, 0), G::WM);
-  const __amdgpu_buffer_rsrc_t zrs = make_rsrc_wave(p.zt + (int64_t)vwave * p.ld_z, (int64_t)zrows * ldz2);
+  const int trows = min(max(p.n - t0, 0), G::WN);
+  const __amdgpu_buffer_rsrc_t zrs =
+      make_rsrc_wave(p.zt == nullptr ? nullptr : p.zt + (int64_t)t0 * p.ld_z, (int64_t)trows * ldz2);
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
-    const int col = n0 + wn * G::WN + ni * 32 + l31;
+    const int col = t0 + ni * 32 + l31;
     // Softcap and the stand-in for rows past V are rare, wave-uniform cases: each sits behind a
     // real scalar branch (the empty asm keeps the compiler from flattening it into per-element
     // selects, which would cost an exp and a reciprocal per logit whether or not a cap is set).
@@ -135,50 +190,126 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
         for (int r = 0; r < 16; ++r)
           if ((vbase + mi * 32 + (r >> 2) * 8 + (r & 3)) >= p.V) g.acc[mi][ni][r] = kNegBig;
     }
-    float mx = kNegBig;
+    // where this lane's eight-entry groups go: token row, then the lane's half of a 16-entry span
+    const bool store = p.zt != nullptr && (t0 + ni * 32) < zt_cols;   // tokens past the live ones are never read
+    const uint32_t voff = (uint32_t)((ni * 32 + l31) * ldz2 + (vwave + lhi * 8) * 2);
+    auto group_off = [&](int mi, int qp) {      // kOob when the lane's eight entries lie past V (V % 8 == 0)
+      return (vwave + mi * 32 + qp * 16 + lhi * 8) < p.V ? voff : kOob;
+    };
+
+    if (MODE == kStatsMax) {
+      float mx = kNegBig;
 #pragma unroll
-    for (int mi = 0; mi < G::MI; ++mi)
+      for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, g.acc[mi][ni][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    float l = 0.f, s = 0.f;
-    const float mxl = mx * kLog2e;
-#pragma unroll
-    for (int mi = 0; mi < G::MI; ++mi)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float z = g.acc[mi][ni][r];
-        const float e = __builtin_amdgcn_exp2f(fmaf(z, kLog2e, -mxl));
-        l += e;
-        s = fmaf(e, z, s);
-      }
-    l += __shfl_xor(l, 32);
-    s += __shfl_xor(s, 32);
-    float lt = 0.f;
-    if (p.inv_t != 1.f) {
-      // The reference takes the log-prob from softmax(z) but the entropy from softmax(z / T)
-      // (train_modules/__init__.py:124-126, :136): a second pair of sums, only when T != 1.
-      asm volatile("");
-      const float kt = kLog2e * p.inv_t, mxt = mx * kt;
-      s = 0.f;
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, g.acc[mi][ni][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      float l = 0.f, s = 0.f;
+      const float mxl = mx * kLog2e;
 #pragma unroll
       for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float z = g.acc[mi][ni][r];
-          const float e = __builtin_amdgcn_exp2f(fmaf(z, kt, -mxt));
-          lt += e;
+          const float e = __builtin_amdgcn_exp2f(fmaf(z, kLog2e, -mxl));
+          l += e;
           s = fmaf(e, z, s);
         }
-      lt += __shfl_xor(lt, 32);
+      l += __shfl_xor(l, 32);
       s += __shfl_xor(s, 32);
-    }
-    if (lhi == 0) {
-      const int64_t o = (int64_t)(tm * 2 + wm) * p.ld_p + col;
-      p.pm[o] = mx;
-      p.pl[o] = l;
-      p.ps[o] = s;
-      if (p.inv_t != 1.f) p.plt[o] = lt;
+      float lt = 0.f;
+      if (p.inv_t != 1.f) {
+        // The reference takes the log-prob from softmax(z) but the entropy from softmax(z / T)
+        // (train_modules/__init__.py:124-126, :136): a second pair of sums, only when T != 1.
+        asm volatile("");
+        const float kt = kLog2e * p.inv_t, mxt = mx * kt;
+        s = 0.f;
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float z = g.acc[mi][ni][r];
+            const float e = __builtin_amdgcn_exp2f(fmaf(z, kt, -mxt));
+            lt += e;
+            s = fmaf(e, z, s);
+          }
+        lt += __shfl_xor(lt, 32);
+        s += __shfl_xor(s, 32);
+      }
+      if (lhi == 0) {
+        const int64_t o = (int64_t)(tm * 2 + wm) * p.ld_p + col;
+        p.pm[o] = mx;
+        p.pl[o] = l;
+        p.ps[o] = s;
+        if (p.inv_t != 1.f) p.plt[o] = lt;
+      }
+      if (store) {
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int qp = 0; qp < 2; ++qp) {
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = g.acc[mi][ni][qp * 8 + j];
+            store_rows8<true>(v, 0xffffffffu, zrs, group_off(mi, qp), (uint32_t)(mi * 32 + qp * 16) * 2);
+          }
+      }
+    } else if (MODE == kStatsExp) {
+      float l = 0.f, s = 0.f;
+      if (store) {
+        const uint32_t keep = (col < p.n && p.mask[col] != 0.f) ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int qp = 0; qp < 2; ++qp) {
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float z = g.acc[mi][ni][qp * 8 + j];
+              const float e = __builtin_amdgcn_exp2f(z * kLog2e);
+              l += e;
+              s = fmaf(e, z, s);
+              v[j] = p.cap > 0.f ? e * (1.f - z * z * inv_cap2) : e;
+            }
+            store_rows8<false>(v, keep, zrs, group_off(mi, qp), (uint32_t)(mi * 32 + qp * 16) * 2);
+          }
+      } else {
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float z = g.acc[mi][ni][r];
+            const float e = __builtin_amdgcn_exp2f(z * kLog2e);
+            l += e;
+            s = fmaf(e, z, s);
+          }
+      }
+      l += __shfl_xor(l, 32);
+      s += __shfl_xor(s, 32);
+      if (lhi == 0) {
+        const int64_t o = (int64_t)(tm * 2 + wm) * p.ld_p + col;
+        p.pl[o] = l;
+        p.ps[o] = s;
+      }
+    } else {   // kStatsGrad
+      const float lse2 = col < p.n ? p.lse[col] * kLog2e : 0.f;
+      const float gneg = col < p.n ? -p.g[col] : 0.f;
+      if (store) {
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int qp = 0; qp < 2; ++qp) {
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float z = g.acc[mi][ni][qp * 8 + j];
+              const float d = gneg * __builtin_amdgcn_exp2f(fmaf(z, kLog2e, -lse2));
+              v[j] = p.cap > 0.f ? d * (1.f - z * z * inv_cap2) : d;
+            }
+            store_rows8<false>(v, gneg != 0.f ? 0xffffffffu : 0u, zrs, group_off(mi, qp),
+                               (uint32_t)(mi * 32 + qp * 16) * 2);
+          }
+      }
     }
     // The sampled token's logit: exactly one lane of one tile holds it.  Few wavefronts have a
     // hit at all (32 tokens x 128 rows out of V), so the register search sits behind a vote.
@@ -196,14 +327,25 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
         if (hit) p.zy[col] = zy;
       }
     }
-    if (p.zt != nullptr && n0 + wn * G::WN + ni * 32 < zt_cols) {   // tokens past the live ones: dZ is never read
-      const uint32_t voff = (uint32_t)((lhi * 4 * p.ld_z + col) * 2);
-#pragma unroll
-      for (int mi = 0; mi < G::MI; ++mi)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          store_b16(f32_to_f16_bits(g.acc[mi][ni][r]), zrs, voff, (uint32_t)(mi * 32 + (r >> 2) * 8 + (r & 3)) * ldz2);
+  }
+}
+
+// One workgroup per tile; RESCUE: a small grid that walks the tile list, and leaves at once unless
+// the range check of the kStatsExp pass failed (state != 0).
+template <int BM, int BN, int MODE, bool RESCUE>
+__global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap map) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  int tm, tn, split;
+  if (RESCUE) {
+    if (__builtin_amdgcn_readfirstlane(*p.state) == 0) return;
+    for (int item = blockIdx.x; item < map.items(); item += gridDim.x) {
+      if (map.tile(item, tm, tn, split)) logits_tile<BM, BN, MODE>(p, tm, tn, smem);
+      __syncthreads();      // the next tile's first LDS writes must not pass this tile's last reads
     }
+  } else {
+    if (MODE == kStatsExp && blockIdx.x == 0 && threadIdx.x == 0) *p.state = 0;
+    if (!map.tile(blockIdx.x, tm, tn, split)) return;
+    logits_tile<BM, BN, MODE>(p, tm, tn, smem);
   }
 }
 
@@ -224,12 +366,29 @@ struct FinalizeArgs {
   float ent_coef, inv_ent_cnt; // entropy bonus (0 = off) and its normaliser
   float* eterm;                // per-token share of the masked mean entropy
   float *ge, *hent;            // [n_pad] coef*mask*inv_ent_cnt*gscale and H_t, or null (no bonus / forward only)
+  // kStatsExp with a backward: row scale of E and the one-hot patch
+  float* rs;                   // [n_pad] -g / sum_v exp(z), or null
+  uint16_t* zt;                // E [n, ld_z]
+  int64_t ld_z;
+  const int32_t* targets;      // chunk origin
+  int V;
+  float cap;
+  int* state;
+  int rescue;                  // kStatsMax launched behind a kStatsExp pass: leave unless state != 0
 };
 
 // block = (64 tokens) x (kFinSlices slices of the partial list)
 constexpr int kFinSlices = 16;
+template <int MODE>
 __global__ __launch_bounds__(64 * kFinSlices) void k_finalize(FinalizeArgs p) {
   __shared__ float sm[kFinSlices][64], sl[kFinSlices][64], ss[kFinSlices][64], st[kFinSlices][64];
+  if (MODE == kStatsMax) {
+    if (p.rescue) {
+      if (__builtin_amdgcn_readfirstlane(*p.state) == 0) return;
+    } else if (blockIdx.x == 0 && threadIdx.x == 0) {
+      *p.state = 1;            // the 16-bit matrix of this chunk will hold dZ itself
+    }
+  }
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int t = blockIdx.x * 64 + tx;
   const bool tempered = p.inv_t != 1.f;   // then s and lt are sums under softmax(z / T)
@@ -237,18 +396,23 @@ __global__ __launch_bounds__(64 * kFinSlices) void k_finalize(FinalizeArgs p) {
   if (t < p.n) {
     for (int q = ty; q < p.parts; q += kFinSlices) {
       const int64_t o = (int64_t)q * p.ld_p + t;
-      const float mq = p.pm[o], lq = p.pl[o], sq = p.ps[o];
-      const float mn = fmaxf(m, mq);
-      const float a = __expf(m - mn), b = __expf(mq - mn);
-      l = l * a + lq * b;
-      if (tempered) {
-        const float at = __expf((m - mn) * p.inv_t), bt = __expf((mq - mn) * p.inv_t);
-        lt = lt * at + p.plt[o] * bt;
-        s = s * at + sq * bt;
+      if (MODE == kStatsExp) {
+        l += p.pl[o];
+        s += p.ps[o];
       } else {
-        s = s * a + sq * b;
+        const float mq = p.pm[o], lq = p.pl[o], sq = p.ps[o];
+        const float mn = fmaxf(m, mq);
+        const float a = __expf(m - mn), b = __expf(mq - mn);
+        l = l * a + lq * b;
+        if (tempered) {
+          const float at = __expf((m - mn) * p.inv_t), bt = __expf((mq - mn) * p.inv_t);
+          lt = lt * at + p.plt[o] * bt;
+          s = s * at + sq * bt;
+        } else {
+          s = s * a + sq * b;
+        }
+        m = mn;
       }
-      m = mn;
     }
   }
   sm[ty][tx] = m; sl[ty][tx] = l; ss[ty][tx] = s; st[ty][tx] = lt;
@@ -257,22 +421,34 @@ __global__ __launch_bounds__(64 * kFinSlices) void k_finalize(FinalizeArgs p) {
   if (t >= p.n) {
     if (p.g != nullptr && t < p.n_pad) p.g[t] = 0.f;
     if (p.ge != nullptr && t < p.n_pad) p.ge[t] = 0.f;
+    if (MODE == kStatsExp && p.rs != nullptr && t < p.n_pad) p.rs[t] = 0.f;
     return;
   }
-  float M = sm[0][tx];
+  float M = 0.f, L = 0.f, S = 0.f, LT = 0.f;
+  if (MODE == kStatsExp) {
 #pragma unroll
-  for (int i = 1; i < kFinSlices; ++i) M = fmaxf(M, sm[i][tx]);
-  float L = 0.f, S = 0.f, LT = 0.f;
+    for (int i = 0; i < kFinSlices; ++i) {
+      L += sl[i][tx];
+      S += ss[i][tx];
+    }
+    // outside the window (or not finite): the sums cannot be trusted; the kStatsMax pass redoes the chunk
+    if (!(L >= kExpSumMin && L <= kExpSumMax)) *p.state = 1;
+  } else {
+    M = sm[0][tx];
 #pragma unroll
-  for (int i = 0; i < kFinSlices; ++i) {
-    const float w = __expf(sm[i][tx] - M);
-    const float wt = tempered ? __expf((sm[i][tx] - M) * p.inv_t) : w;
-    L += sl[i][tx] * w;
-    S += ss[i][tx] * wt;
-    LT += st[i][tx] * wt;
+    for (int i = 1; i < kFinSlices; ++i) M = fmaxf(M, sm[i][tx]);
+#pragma unroll
+    for (int i = 0; i < kFinSlices; ++i) {
+      const float w = __expf(sm[i][tx] - M);
+      const float wt = tempered ? __expf((sm[i][tx] - M) * p.inv_t) : w;
+      L += sl[i][tx] * w;
+      S += ss[i][tx] * wt;
+      LT += st[i][tx] * wt;
+    }
   }
   const float lse = M + __logf(L);
-  const float logp = (p.zy[t] - lse) * p.inv_t;     // division after the log-softmax (:124-126)
+  const float zy = p.zy[t];
+  const float logp = (zy - lse) * p.inv_t;     // division after the log-softmax (:124-126)
   p.lse[t] = lse;
   p.logp[t] = logp;
   // entropy of softmax(z / T): log sum e^(z/T) - sum p z / T  (reference adds 1e-9 inside the log)
@@ -298,7 +474,34 @@ __global__ __launch_bounds__(64 * kFinSlices) void k_finalize(FinalizeArgs p) {
     g = active ? -mk * p.inv_tv * adv * ratio : 0.f;
   }
   p.term[t] = term;
-  if (p.g != nullptr) p.g[t] = g * p.gscale * p.inv_t;   // dlogp/dz = (onehot - softmax(z)) / T
+  g *= p.gscale * p.inv_t;                     // dlogp/dz = (onehot - softmax(z)) / T
+  if (p.g != nullptr) p.g[t] = g;
+  if (MODE == kStatsExp && p.rs != nullptr) {
+    // dZ[t, v] = g (onehot - e_v / L) cap'_v = (-g / L) (E[t, v] - onehot * L * cap'_y)
+    p.rs[t] = -g / L;
+    if (mk != 0.f) {                           // masked tokens keep their zero row
+      const int y = clamp_target(p.targets[t], p.V);
+      const float capf = p.cap > 0.f ? 1.f - (zy / p.cap) * (zy / p.cap) : 1.f;
+      p.zt[(int64_t)t * p.ld_z + y] = f32_to_bf16((__builtin_amdgcn_exp2f(zy * kLog2e) - L) * capf);
+    }
+  }
+}
+
+// rs[t] * hidden[t, :] in bf16: the token-side operand of the dW product when the 16-bit matrix
+// holds E (one thread = 8 columns)
+__global__ __launch_bounds__(256) void k_scale_hidden(const uint16_t* hid, int64_t ld_hid, const float* rs, int n,
+                                                      int H, uint16_t* hs) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int h8 = H >> 3;
+  if (i >= (int64_t)n * h8) return;
+  const int row = (int)(i / h8), c = (int)(i % h8) * 8;
+  const float r = rs[row];
+  const u32x4 in = *(const u32x4*)(hid + (int64_t)row * ld_hid + c);
+  u32x4 out;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    out[j] = pack_bf16(r * __uint_as_float(in[j] << 16), r * __uint_as_float(in[j] & 0xffff0000u));
+  *(u32x4*)(hs + (int64_t)row * H + c) = out;
 }
 
 // dloss/dlogp from a saved forward (separate backward entry point)
@@ -323,6 +526,21 @@ __global__ __launch_bounds__(256) void k_coeff_from_saved(const float* logp, con
     }
   }
   g[t] = out * gscale;
+}
+
+// kStatsGrad: the sampled token's entry of dZ, g (1 - p_y) cap'_y, replaces the -g p_y cap'_y the
+// epilogue wrote there; marks the 16-bit matrix as dZ.
+__global__ __launch_bounds__(256) void k_patch_grad(uint16_t* zt, int64_t ld_z, const float* zy, const float* lse,
+                                                    const float* g, const int32_t* targets, int n, int V, float cap,
+                                                    int* state) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t == 0) *state = 1;
+  if (t >= n) return;
+  const float gt = g[t];
+  if (gt == 0.f) return;                        // the row is all zeros
+  const float z = zy[t];
+  const float capf = cap > 0.f ? 1.f - (z / cap) * (z / cap) : 1.f;
+  zt[(int64_t)t * ld_z + clamp_target(targets[t], V)] = f32_to_bf16(gt * (1.f - __expf(z - lse[t])) * capf);
 }
 
 // Deterministic single-workgroup sums: loss[1] = masked mean entropy, loss[0] = sum of the
@@ -353,71 +571,59 @@ __global__ __launch_bounds__(1024) void k_reduce_loss(const float* term, const f
 
 // ----------------------------------------------------------------------------- dZ
 struct DzArgs {
-  uint16_t* zt;        // [V, ld_z] in: capped logits^T (half); out: dZ^T (bf16)
+  uint16_t* zt;        // [n, ld_z] in: capped logits (half); out: dZ (bf16)
   int64_t ld_z;
   const float *lse, *g;    // chunk-local (lse valid for t < n, g for t < n_pad)
   const float *ge, *hent;  // chunk-local entropy-bonus coefficient and H_t, or null
   const int32_t* targets;  // chunk origin
-  int V, n, n_pad;
+  int V, n;
   float cap;
   const int* n_live;   // see live_pad
   int c0;
+  const int* state;
+  int rescue;          // launched behind a kStatsExp pass: leave unless state != 0
 };
 
-// Streaming, in place.  Block = 256 tokens (32 threads x 8) by kDzRows vocab rows (8 row-lanes x
-// 8 steps per pass): every wavefront instruction moves two full 512-byte row segments, and the
-// per-token constants are loaded once per thread.  Tokens at or beyond n (chunk padding) become
-// exact zeros.  The rows per block are chosen so that the launch is bound by HBM, not by the rate
-// at which workgroups can be dispatched.
-constexpr int kDzRows = 512;
+// Streaming, in place, after a kStatsMax pass.  A workgroup takes whole token rows: the per-token
+// constants are loaded once, every thread moves 16 bytes per step and the 256 threads cover 4 KB
+// of the row at a time.
 __global__ __launch_bounds__(256) void k_dz(DzArgs p) {
-  const int cx = threadIdx.x & 31, ry = threadIdx.x >> 5;
-  const int t0 = blockIdx.y * 256 + cx * 8;      // vocab blocks vary fastest: whatever part of the
-  const int vblock = blockIdx.x * kDzRows;        // tokens is live, its work spreads over all XCDs
-  if (t0 >= live_pad(p.n_live, p.c0, p.n_pad)) return;
+  if (p.rescue && __builtin_amdgcn_readfirstlane(*p.state) == 0) return;
+  const int lim = min(p.n, live_pad(p.n_live, p.c0, (p.n + 255) & ~255));
   const float inv_cap2 = p.cap > 0.f ? 1.f / (p.cap * p.cap) : 0.f;
   const bool bonus = p.ge != nullptr;
-  float lse[8], g[8], ge[8], hent[8];
-  int y[8];
+  for (int t = blockIdx.x; t < lim; t += gridDim.x) {
+    const float lse = p.lse[t] * kLog2e, g = p.g[t];
+    const float ge = bonus ? p.ge[t] : 0.f, hent = bonus ? p.hent[t] : 0.f;
+    const int y = clamp_target(p.targets[t], p.V);
+    const bool dead = !(g != 0.f) && !(ge != 0.f);   // masked token: exactly zero, whatever z holds
+    uint16_t* row = p.zt + (int64_t)t * p.ld_z;
+    for (int v0 = threadIdx.x * 8; v0 < p.V; v0 += 256 * 8) {
+      u32x4 out = {0u, 0u, 0u, 0u};
+      if (!dead) {
+        const u32x4 in = *(const u32x4*)(row + v0);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int t = t0 + i;
-    const bool in = t < p.n;
-    lse[i] = in ? p.lse[t] * kLog2e : 0.f;
-    g[i] = in ? p.g[t] : 0.f;
-    y[i] = in ? clamp_target(p.targets[t], p.V) : -1;
-    ge[i] = (bonus && in) ? p.ge[t] : 0.f;
-    hent[i] = (bonus && in) ? p.hent[t] : 0.f;
-  }
-  for (int v0 = vblock; v0 < min(vblock + kDzRows, p.V); v0 += 64)
-#pragma unroll
-  for (int step = 0; step < 8; ++step) {
-    const int v = v0 + step * 8 + ry;
-    if (v >= p.V) break;
-    uint16_t* ptr = p.zt + (int64_t)v * p.ld_z + t0;
-    const u32x4 in = *(const u32x4*)ptr;
-    u32x4 out;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t w = in[i >> 1];
-      const float z = f16_bits_to_f32((uint16_t)((i & 1) ? (w >> 16) : (w & 0xffffu)));
-      const float t2 = fmaf(z, kLog2e, -lse[i]);          // log2 p
-      const float pr = __builtin_amdgcn_exp2f(t2);
-      float d = (v == y[i]) ? 1.f - pr : -pr;
-      d *= g[i];
-      if (bonus) d = fmaf(ge[i] * pr, fmaf(t2, 0.6931471805599453f, hent[i]), d);   // coef * p * (log p + H)
-      if (p.cap > 0.f) d *= 1.f - z * z * inv_cap2;
-      if (!(g[i] != 0.f) && !(ge[i] != 0.f)) d = 0.f;   // masked or padding token: exactly zero, whatever z holds
-      const uint32_t b = f32_to_bf16(d);
-      if (i & 1) out[i >> 1] |= b << 16; else out[i >> 1] = b;
+        for (int i = 0; i < 8; ++i) {
+          const uint32_t w = in[i >> 1];
+          const float z = f16_bits_to_f32((uint16_t)((i & 1) ? (w >> 16) : (w & 0xffffu)));
+          const float t2 = fmaf(z, kLog2e, -lse);          // log2 p
+          const float pr = __builtin_amdgcn_exp2f(t2);
+          float d = (v0 + i == y) ? 1.f - pr : -pr;
+          d *= g;
+          if (bonus) d = fmaf(ge * pr, fmaf(t2, 0.6931471805599453f, hent), d);   // coef * p * (log p + H)
+          if (p.cap > 0.f) d *= 1.f - z * z * inv_cap2;
+          const uint32_t b = f32_to_bf16(d);
+          if (i & 1) out[i >> 1] |= b << 16; else out[i >> 1] = b;
+        }
+      }
+      *(u32x4*)(row + v0) = out;
     }
-    *(u32x4*)ptr = out;
   }
 }
 
 // ----------------------------------------------------------------------------- backward products
 struct DhArgs {
-  const __bf16* dzt;  // [V, ld_z] dZ^T of the chunk
+  const __bf16* dzt;  // [n, ld_z] E or dZ of the chunk (see StatsMode)
   const __bf16* w;    // [H, ld_w]
   int64_t ld_z, ld_w;
   int n, n_pad, H, V;
@@ -427,11 +633,13 @@ struct DhArgs {
   float* part;        // [splits, n_pad, H] fp32 partial sums (splits > 1)
   const int* n_live;  // see live_pad
   int c0;
+  const float* rs;    // [n_pad] row scale, applied when state == 0
+  const int* state;
 };
 
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
-  using G = GemmTN<BM, BN, kKRow, kRowK>;
+  using G = GemmTN<BM, BN, kRowK, kRowK>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   // Only token tiles that hold live tokens are walked: the tile list is rebuilt for that many
   // rows of tiles, so that the live work spreads evenly over the XCDs (ids past its end leave).
@@ -442,26 +650,34 @@ __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
   const int k0 = split * p.k_per_split;
   const int klen = min(p.V - k0, p.k_per_split);
   G g;
-  g.run(p.dzt + (int64_t)k0 * p.ld_z + m0, p.n_pad - m0, p.ld_z, p.w + (int64_t)n0 * p.ld_w + k0, p.H - n0,
-        p.ld_w, klen, smem);
+  g.run(p.dzt + (int64_t)m0 * p.ld_z + k0, p.n - m0, p.ld_z, p.w + (int64_t)n0 * p.ld_w + k0, p.H - n0, p.ld_w,
+        klen, smem);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps descriptors in SGPRs
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
   const int row0 = m0 + wm * G::WM;                       // first token row of this wavefront
   const int rows = min(max(p.n - row0, 0), G::WM);        // rows at or past n are dropped
   if (p.splits == 1) {
+    const bool scaled = __builtin_amdgcn_readfirstlane(*p.state) == 0;
     const uint32_t ld2 = (uint32_t)p.ld_dh * 2;
     const __amdgpu_buffer_rsrc_t rs = make_rsrc_wave(p.dh + (int64_t)row0 * p.ld_dh, (int64_t)rows * ld2);
+    const __amdgpu_buffer_rsrc_t srs = make_rsrc_wave(p.rs + row0, (int64_t)rows * 4);   // rows past n read 0
 #pragma unroll
-    for (int ni = 0; ni < G::NI; ++ni) {
-      const int col = n0 + wn * G::WN + ni * 32 + l31;
-      const uint32_t voff = col < p.H ? (uint32_t)(lhi * 4 * ld2 + col * 2) : kOob;
+    for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
-      for (int mi = 0; mi < G::MI; ++mi)
+      for (int q = 0; q < 4; ++q) {
+        // the four consecutive token rows of this lane in the 8-row group q of block mi
+        f32x4 sc = {1.f, 1.f, 1.f, 1.f};
+        if (scaled) sc = load_b128(srs, (uint32_t)(lhi * 16), (uint32_t)(mi * 32 + q * 8) * 4);
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          store_b16(f32_to_bf16(g.acc[mi][ni][r]), rs, voff, (uint32_t)(mi * 32 + (r >> 2) * 8 + (r & 3)) * ld2);
-    }
+        for (int ni = 0; ni < G::NI; ++ni) {
+          const int col = n0 + wn * G::WN + ni * 32 + l31;
+          const uint32_t voff = col < p.H ? (uint32_t)(lhi * 4 * ld2 + col * 2) : kOob;
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            store_b16(f32_to_bf16(g.acc[mi][ni][q * 4 + j] * sc[j]), rs, voff, (uint32_t)(mi * 32 + q * 8 + j) * ld2);
+        }
+      }
   } else {
     const uint32_t ld4 = (uint32_t)p.H * 4;
     const __amdgpu_buffer_rsrc_t rs =
@@ -479,15 +695,18 @@ __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
   }
 }
 
-// dh[row, :] = bf16(sum over splits of part[s, row, :]), fixed order.
+// dh[row, :] = bf16(scale * sum over splits of part[s, row, :]), fixed order; scale = rs[row] when the
+// 16-bit matrix held E (state == 0), else 1.
 __global__ __launch_bounds__(256) void k_dhidden_reduce(const float* part, int splits, int n, int n_pad, int H,
-                                                        uint16_t* dh, int64_t ld_dh) {
+                                                        uint16_t* dh, int64_t ld_dh, const float* rs,
+                                                        const int* state) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;   // one thread = 4 columns
   const int h4 = H / 4;
   if (i >= (int64_t)n * h4) return;
   const int row = (int)(i / h4), c = (int)(i % h4) * 4;
   f32x4 a = *(const f32x4*)(part + (int64_t)row * H + c);
   for (int s = 1; s < splits; ++s) a += *(const f32x4*)(part + ((int64_t)s * n_pad + row) * H + c);
+  if (*state == 0) a *= rs[row];
   uint16_t* o = dh + (int64_t)row * ld_dh + c;
   const uint32_t lo = f32_to_bf16(a[0]) | ((uint32_t)f32_to_bf16(a[1]) << 16);
   const uint32_t hi = f32_to_bf16(a[2]) | ((uint32_t)f32_to_bf16(a[3]) << 16);
@@ -495,29 +714,35 @@ __global__ __launch_bounds__(256) void k_dhidden_reduce(const float* part, int s
 }
 
 struct DwArgs {
-  const __bf16* dzt;   // [V, ld_z] dZ^T of the chunk
+  const __bf16* dzt;   // [n, ld_z] E or dZ of the chunk
   const __bf16* hid;   // chunk origin [n, ld_hid]
+  const __bf16* hs;    // [n, H]: rs * hidden, the token-side operand while state == 0
   int64_t ld_z, ld_hid;
-  int H, V, n;         // n = tokens of the chunk (dZ^T holds zeros from n up to its padded width)
+  int H, V, n;         // n = tokens of the chunk
   float* dw;           // [H, ld_dw] f32
   int64_t ld_dw;
   int accumulate;
   const int* n_live;   // see live_pad
   int c0;
+  const int* state;
 };
 
 // Tile of dW^T: rows = vocab (MFMA row direction), columns = hidden (lanes).  A lane's four
 // consecutive accumulator rows are four consecutive floats of one dW row: 16-byte accesses.
+// Both operands are token-major in memory, so both go through the transposing LDS read.
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
-  using G = GemmTN<BM, BN, kRowK, kKRow>;
+  using G = GemmTN<BM, BN, kKRow, kKRow>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   int tm, tn, split;
   if (!map.tile(blockIdx.x, tm, tn, split)) return;
   const int m0 = tm * BM, n0 = tn * BN;
   G g;
   const int kn = min(p.n, live_pad(p.n_live, p.c0, (p.n + 255) & ~255));   // tokens past the live ones have dZ = 0
-  g.run(p.dzt + (int64_t)m0 * p.ld_z, p.V - m0, p.ld_z, p.hid + n0, p.H - n0, p.ld_hid, kn, smem);
+  const bool scaled = __builtin_amdgcn_readfirstlane(*p.state) == 0;
+  const __bf16* tok = scaled ? p.hs : p.hid;
+  const int64_t ld_tok = scaled ? (int64_t)p.H : p.ld_hid;
+  g.run(p.dzt + m0, p.V - m0, p.ld_z, tok + n0, p.H - n0, ld_tok, kn, smem);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps descriptors in SGPRs
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;

@@ -184,7 +184,42 @@ def test_forward_only_and_separate_backward_match_fused():
         C.byref(p.desc), _ptr(p.hidden), _ptr(p.w), _ptr(p.targets), _ptr(p.old), _ptr(p.adv), _ptr(p.mask),
         _ptr(p.lse), _ptr(p.logp), _ptr(dh2), _ptr(dw2), _ptr(ws), ws.numel(), p.stream()))
     torch.cuda.synchronize()
-    assert torch.equal(dh, dh2) and torch.equal(dw, dw2)
+    # the fused pass forms dZ as rs * E (E = exp(z) in bf16), the separate backward rounds dZ itself
+    # to bf16: same gradient, different roundings
+    ref = O.grpo_loss(hid.float().numpy(), w.float().numpy(), y.numpy(), old.numpy(), adv.numpy(), mask.numpy())
+    for got_h, got_w in ((dh, dw), (dh2, dw2)):
+        assert _rel(got_h.float().cpu().numpy(), ref["d_hidden"]) <= GRAD_RTOL
+        assert _rel(got_w[:, :1032].cpu().numpy(), ref["d_lm_head"]) <= GRAD_RTOL
+    assert _rel(dh2.float().cpu().numpy(), dh.float().cpu().numpy()) <= 1e-2
+    assert _rel(dw2.cpu().numpy(), dw.cpu().numpy()) <= 1e-2
+
+
+@pytest.mark.parametrize("shift", [100.0, -100.0])
+def test_logits_outside_the_exp_window_take_the_rescue_pass(shift):
+    """The fast statistics sum exp(z) without a running maximum and are valid while logsumexp stays
+    within about +-60.  Here one chunk of three has every logit shifted by +-100 (a rank-one term in
+    the hidden states): its range check fails on the device and the running-maximum pass redoes that
+    chunk, the other chunks keep the fast results; all of it must match the oracle."""
+    n, h, v, b = 768, 64, 1000, 3
+    hid, w, y, adv, mask = _case(21, n, h, v, b)
+    w = w.float()
+    w[0, :] = 1.0                                  # hidden[:, 0] becomes a common offset of the logits
+    hid = hid.float()
+    hid[:, 0] = 0.0
+    hid[256:512, 0] = shift                        # second chunk of 256 tokens only
+    hid, w = hid.to(torch.bfloat16), w.to(torch.bfloat16)
+    old = _old_from(_ref_logp(hid, w, y), 22)
+    met, dh, dw, ref = _check(hid, w, y, old, adv, mask, seq_shape=(b, n // b), chunk_tokens=256,
+                              epsilon_low=0.2, epsilon_high=0.28)
+    assert abs(ref["lse"][300] - shift) < 15 and abs(ref["lse"][10]) < 15
+    # forward-only takes the same decision per chunk: bit-identical outputs
+    import mllm_jax_amd as M
+    d = _dev()
+    with torch.no_grad():
+        fwd = M.grpo_fused_loss(hid.to(d), w.to(d), y.to(d), old.to(d), adv.to(d), mask.to(d), chunk_tokens=256,
+                                epsilon_low=0.2, epsilon_high=0.28, return_token_entropy=True)
+    np.testing.assert_array_equal(fwd["per_token_logps"].cpu().numpy().reshape(-1), met["per_token_logps"].reshape(-1))
+    np.testing.assert_array_equal(fwd["token_entropy"].cpu().numpy().reshape(-1), met["token_entropy"].reshape(-1))
 
 
 def test_deterministic_and_accumulate():
