@@ -101,6 +101,22 @@ int mj_grpo_forward(const MjGrpoDesc* desc, const void* hidden, const void* lm_h
                     const float* mask, float* logp, float* lse, float* token_entropy,
                     float* loss, void* workspace, size_t workspace_bytes, void* stream);
 
+/* mj_grpo_forward without a workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops that score log-probs, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  The statistics that mj_grpo_forward keeps in the
+ * caller's workspace live in a static device array of MJ_GRPO_NOALLOC_SCRATCH_BYTES that every device
+ * the library runs on holds until the process ends; the call allocates and frees nothing.
+ * chunk_tokens == 0 picks the largest chunk that fits (at most 16384 tokens).  Shapes whose workspace
+ * does not fit even with 256-token chunks (12 bytes per token plus 6 * ceil(V/256) * 4 bytes per
+ * token of a chunk) are refused with MJ_GRPO_ERR_WORKSPACE.  All calls on one device share the
+ * array: calls that overlap on a device (two streams, two threads) race; serialise them.  Outputs
+ * are those of mj_grpo_forward bit for bit. */
+#define MJ_GRPO_NOALLOC_SCRATCH_BYTES (32u << 20)
+int mj_grpo_forward_noalloc(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
+                            const int32_t* targets, const float* old_logp, const float* advantages,
+                            const float* mask, float* logp, float* lse, float* token_entropy,
+                            float* loss, void* stream);
+
 /* Forward and backward in one pass (executes 6*N*H*V flop).  Replaces
  * jax.value_and_grad(loss_fn) of plugins/training/update/train_step.py:15-24 restricted to
  * the lm_head + loss part: besides the forward outputs it writes

@@ -9,6 +9,7 @@
 #include <stdio.h>
 
 #include <initializer_list>
+#include <mutex>
 #include <new>
 
 #include "mj_grpo_kernels.hpp"
@@ -494,6 +495,73 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
                      size_t workspace_bytes, void* stream) {
   return run(kBackwardOnly, desc, hidden, lm_head, targets, old_logp, advantages, mask, nullptr, nullptr,
              nullptr, nullptr, lse, logp, d_hidden, d_lm_head, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"
+
+// ---- forward without a caller workspace: the workspace is a static device array
+namespace {
+constexpr size_t kScratchBytes = (size_t)MJ_GRPO_NOALLOC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+namespace {
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};   // device address of `scratch` on each device, once looked up
+
+// The array's name is only a host-side handle; this returns the current device's copy of it.
+int scratch_address(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(MJ_GRPO_ERR_UNSUPPORTED, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return fail(MJ_GRPO_ERR_HIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return MJ_GRPO_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int mj_grpo_forward_noalloc(const MjGrpoDesc* desc, const void* hidden, const void* lm_head, const int32_t* targets,
+                            const float* old_logp, const float* advantages, const float* mask, float* logp,
+                            float* lse, float* token_entropy, float* loss, void* stream) {
+  if (desc == nullptr) return fail(MJ_GRPO_ERR_NULL, "desc is NULL");
+  MjGrpoDesc d = *desc;
+  Plan p;
+  int rc;
+  if (d.chunk_tokens > 0) {
+    if ((rc = make_plan(&d, &p))) return rc;
+  } else {
+    // the largest chunk (a multiple of 256 tokens) whose statistics fit the static array
+    int64_t lo = 1, hi = (d.n_tokens + 255) / 256;   // in units of 256 tokens
+    if (hi > 64) hi = 64;
+    d.chunk_tokens = 256;
+    if ((rc = make_plan(&d, &p))) return rc;
+    while (p.total_fwd <= kScratchBytes && lo < hi) {
+      const int64_t mid = (lo + hi + 1) / 2;
+      MjGrpoDesc t = d;
+      t.chunk_tokens = mid * 256;
+      Plan q;
+      if ((rc = make_plan(&t, &q))) return rc;
+      if (q.total_fwd <= kScratchBytes) { lo = mid; d = t; p = q; } else { hi = mid - 1; }
+    }
+  }
+  if (p.total_fwd > kScratchBytes)
+    return fail(MJ_GRPO_ERR_WORKSPACE,
+                "this shape needs %zu bytes of forward workspace with %lld-token chunks; the static array holds %zu "
+                "(use mj_grpo_forward with a caller workspace)", p.total_fwd, (long long)p.chunk, kScratchBytes);
+  void* ws = nullptr;
+  if ((rc = scratch_address(&ws))) return rc;
+  return run(kForward, &d, hidden, lm_head, targets, old_logp, advantages, mask, logp, lse, token_entropy, loss,
+             nullptr, nullptr, nullptr, nullptr, ws, kScratchBytes, stream);
 }
 
 }  // extern "C"
