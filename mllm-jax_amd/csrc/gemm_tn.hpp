@@ -190,7 +190,14 @@ struct Operand {
   }
 };
 
-template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK, int WAVES_M = 2, int WAVES_N = 2>
+template <int V>
+struct IntTag { static constexpr int value = V; };
+
+// DEPTH: slices in flight between global memory and the LDS.  1: the loads of slice k+2 are issued
+// during slice k and written to the LDS during slice k+1 (one slice of math to land).  2: a second
+// set of staging registers; the loads of slice k+3 are issued during slice k and written during
+// slice k+2 (two slices to land) -- for shapes whose operands come from HBM on every slice.
+template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK, int DEPTH = 1, int WAVES_M = 2, int WAVES_N = 2>
 struct GemmTN {
   static_assert(BM % 32 == 0 && BN % 32 == 0, "tile sides are multiples of 32");
   static constexpr int kWavesM = WAVES_M, kWavesN = WAVES_N;
@@ -213,6 +220,10 @@ struct GemmTN {
   // ld*: elements between rows (kRowK) or between k-rows (kKRow); K: k extent from the origin.
   MJ_DEV void run(const __bf16* A, int rows_a, int64_t lda, const __bf16* B, int rows_b,
                   int64_t ldb, int K, char* smem) {
+    if (DEPTH == 2) {
+      run_deep(A, rows_a, lda, B, rows_b, ldb, K, smem);
+      return;
+    }
     const int wave = threadIdx.x >> 6;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     OpA a;
@@ -294,6 +305,99 @@ struct GemmTN {
       __builtin_amdgcn_sched_barrier(0);
       kstep(1, kt + 1, 0, kt, LPS);
     }
+  }
+
+  // DEPTH == 2 (see the struct's comment).  Iteration kt stores slice kt+1 from staging set
+  // (kt+1) & 1 and refills that set with slice kt+3; the loop is unrolled by two so that the set
+  // index is a compile-time constant.
+  MJ_DEV void run_deep(const __bf16* A, int rows_a, int64_t lda, const __bf16* B, int rows_b, int64_t ldb,
+                       int K, char* smem) {
+    const int wave = threadIdx.x >> 6;
+    const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+    OpA a;
+    OpB b;
+    a.init(A, rows_a, lda, K, wm * WM);
+    b.init(B, rows_b, ldb, K, wn * WN);
+
+    u32x4 staged[2][LPS];
+    auto load_one = [&](auto set, int slice, int j) {
+      constexpr int S = decltype(set)::value;
+      if (j < A_LD) staged[S][j] = a.load(slice, j);
+      else staged[S][j] = b.load(slice, j - A_LD);
+    };
+    auto store_one = [&](auto set, int slice, int j) {
+      constexpr int S = decltype(set)::value;
+      char* stage = smem + (slice & 1) * kStageBytes;
+      if (j < A_LD) a.store(stage, j, staged[S][j]);
+      else b.store(stage + OpA::kBytes, j - A_LD, staged[S][j]);
+    };
+    bf16x8 fa[2][MI], fb[2][NI];
+    auto read_one = [&](int slice, int ks, int buf, int g) {
+      const char* stage = smem + (slice & 1) * kStageBytes;
+      if (g < MI) fa[buf][g] = a.frag(stage, g, ks);
+      else fb[buf][g - MI] = b.frag(stage + OpA::kBytes, g - MI, ks);
+    };
+    constexpr int G = MI + NI, T = MI * NI;
+    auto kstep = [&](auto set, int buf, int next_slice, int next_ks, int kt, int first) {
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        if (first + g < LPS) {
+          store_one(set, kt + 1, first + g);
+          load_one(set, kt + 3, first + g);
+        }
+        read_one(next_slice, next_ks, buf ^ 1, g);
+#pragma unroll
+        for (int p = g * T / G; p < (g + 1) * T / G; ++p)
+          acc[p / NI][p % NI] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][p / NI], fb[buf][p % NI],
+                                                                        acc[p / NI][p % NI], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    auto iteration = [&](auto set, int kt) {
+      a.slice_begin(kt + 3);
+      b.slice_begin(kt + 3);
+      kstep(set, 0, kt, 1, kt, 0);
+      kstep(set, 1, kt, 2, kt, G);
+      kstep(set, 0, kt, 3, kt, 2 * G);
+      wait_lgkmcnt0();                  // own reads of slice kt and writes of slice kt+1 are done
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      kstep(set, 1, kt + 1, 0, kt, LPS);
+    };
+
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+
+    const int KT = (K + kBK - 1) / kBK;
+    a.slice_begin(0);
+    b.slice_begin(0);
+#pragma unroll
+    for (int j = 0; j < LPS; ++j) load_one(IntTag<0>(), 0, j);
+    a.slice_begin(1);
+    b.slice_begin(1);
+#pragma unroll
+    for (int j = 0; j < LPS; ++j) load_one(IntTag<1>(), 1, j);
+    a.slice_begin(2);
+    b.slice_begin(2);
+#pragma unroll
+    for (int j = 0; j < LPS; ++j) {
+      store_one(IntTag<0>(), 0, j);
+      load_one(IntTag<0>(), 2, j);
+    }
+    wait_lgkmcnt0();
+    __builtin_amdgcn_s_barrier();       // slice 0 is in LDS, slices 1 and 2 are on their way to the registers
+#pragma unroll
+    for (int g = 0; g < G; ++g) read_one(0, 0, 0, g);
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+      iteration(IntTag<1>(), kt);       // even kt: slice kt+1 waits in set 1
+      iteration(IntTag<0>(), kt + 1);
+    }
+    if (kt < KT) iteration(IntTag<1>(), kt);
   }
 };
 

@@ -732,7 +732,7 @@ struct DwArgs {
 // Both operands are token-major in memory, so both go through the transposing LDS read.
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
-  using G = GemmTN<BM, BN, kKRow, kKRow>;
+  using G = GemmTN<BM, BN, kKRow, kKRow, 2>;   // two slices in flight: measured 2-3% faster here, not in the other products
   extern __shared__ __attribute__((aligned(16))) char smem[];
   int tm, tn, split;
   if (!map.tile(blockIdx.x, tm, tn, split)) return;
