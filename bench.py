@@ -25,9 +25,9 @@ PEAK_HBM_GBS = 8000.0
 # a plain 1 GiB device copy (x2.00 fetch, x1.00 write); summary in profiles/.  Keyed by
 # (config index, kernel); None for workloads that were not counted.
 MEASURED_TRAFFIC_BYTES = {          # default chunk (16384 tokens: one launch of each kernel per step)
-    (2, "k_logits_stats"): 32.57e9,
-    (2, "k_dhidden"): 51.75e9,
-    (2, "k_dw"): 30.53e9,
+    (2, "k_logits_stats"): 32.56e9,
+    (2, "k_dhidden"): 34.43e9,
+    (2, "k_dw"): 37.24e9,
 }
 
 
@@ -131,6 +131,38 @@ class _SmiSampler:
         return out
 
 
+def _mfma_probe(torch, _lib, dev):
+    import ctypes as C
+    lib = _lib.load()
+    out = torch.empty(1024 * 256, dtype=torch.float32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    res = {"metric": "mfma_only_bf16_tflops", "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS,
+           "kernel": "k_probe_mfma: 1024 workgroups x 4 wavefronts x (4x4 blocks of v_mfma_f32_32x32x16_bf16), "
+                     "operands in registers, two operand sets alternating"}
+    for name in ("random", "zero"):
+        ops = torch.randn(512 * 1024, device=dev).to(torch.bfloat16) if name == "random" \
+            else torch.zeros(512 * 1024, dtype=torch.bfloat16, device=dev)
+        flop = C.c_double(0.0)
+        launch = lambda: _lib.check(lib.mj_grpo_probe_mfma(ops.data_ptr(), out.data_ptr(), 1024, 20000, C.byref(flop), st))
+        launch()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        with _SmiSampler() as smi:
+            time.sleep(0.6)
+            t0 = time.perf_counter()
+            e0.record()
+            reps = 60                      # ~50 ms per launch: about 3 s of sustained MFMA work
+            for _ in range(reps):
+                launch()
+            e1.record()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+        ms = e0.elapsed_time(e1) / reps
+        res[name] = {"ms_per_launch": round(ms, 3), "tflops": round(flop.value / ms / 1e9, 1),
+                     "frac_of_peak": round(flop.value / ms / 1e9 / PEAK_BF16_TFLOPS, 4), "smi": smi.summary(t0, t1)}
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -145,6 +177,10 @@ def main() -> int:
     ap.add_argument("--zero-operands", action="store_true",
                     help="time the same launches with all-zero hidden and lm_head (MFMA power depends on the operand "
                          "data; the loss value is then meaningless)")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="instead of the loss: run the library's MFMA-only loop (no memory traffic) for ~3 s each with "
+                         "random and with all-zero bf16 operands and print what the matrix cores sustain under the "
+                         "power cap, with amd-smi power / clock samples")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-masked", action="store_true",
@@ -172,6 +208,9 @@ def main() -> int:
         print("bench.py: no GPU visible; the fused loss has no CPU path", file=sys.stderr)
         return 3
     dev = torch.device("cuda:0")
+    if args.mfma_probe:
+        print(json.dumps(_mfma_probe(torch, _lib, dev)), flush=True)
+        return 0
     cfg = M.CONFIGS[args.config]
     kw = dict(epsilon_low=cfg.eps_low, epsilon_high=cfg.eps_high, final_logit_softcap=cfg.softcap,
               chunk_tokens=args.chunk_tokens or None, dhidden_splits=args.dhidden_splits)

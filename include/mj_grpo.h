@@ -186,6 +186,15 @@ enum {
 int mj_grpo_profile_begin(int max_launches);
 int mj_grpo_profile_end(double* total_ms /* [MJ_GRPO_K_COUNT] */, int* launches /* [MJ_GRPO_K_COUNT] */);
 
+/* Measurement support (no counterpart in the reference): an MFMA-only loop with the register tile
+ * of the product kernels (4 wavefronts x 16 blocks of v_mfma_f32_32x32x16_bf16 per workgroup, no
+ * memory traffic while it runs).  operands: 1 MiB of bf16 data on the device (what the multipliers
+ * see: random values or zeros); out: workgroups * 256 floats; *flop receives the flop executed.
+ * Timed by the caller with events on `stream`; shows what the matrix cores sustain under the
+ * GPU's power cap for a given operand data pattern. */
+int mj_grpo_probe_mfma(const void* operands, float* out, int workgroups, int iters, double* flop,
+                       void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -16,7 +16,7 @@ FLAG_SFT = 1 << 1
 FLAG_SKIP_MASKED = 1 << 2
 
 EXPORTS = ("mj_grpo_version", "mj_grpo_last_error", "mj_grpo_workspace_bytes", "mj_grpo_forward",
-           "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_forward_noalloc", "mj_grpo_profile_begin", "mj_grpo_profile_end",
+           "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_forward_noalloc", "mj_grpo_probe_mfma", "mj_grpo_profile_begin", "mj_grpo_profile_end",
            "mj_grpo_group_advantages", "mj_grpo_advantages", "mj_grpo_gae", "mj_rmsnorm_forward", "mj_sample_logits", "mj_sample_top_k", "mj_rmsnorm_workspace_bytes", "mj_rmsnorm_backward")
 
 KERNEL_NAMES = ("k_logits_stats", "k_finalize", "k_dz", "k_dhidden", "k_dhidden_reduce", "k_dw",
@@ -59,6 +59,7 @@ def load() -> C.CDLL:
     lib.mj_grpo_workspace_bytes.argtypes = [dp, C.POINTER(sz), C.POINTER(sz)]
     lib.mj_grpo_forward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp, sz, vp]
     lib.mj_grpo_forward_noalloc.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp]
+    lib.mj_grpo_probe_mfma.argtypes = [vp, fp, C.c_int, C.c_int, C.POINTER(C.c_double), vp]
     lib.mj_grpo_forward_backward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp, fp, vp, sz, vp]
     lib.mj_grpo_backward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, vp, fp, vp, sz, vp]
     lib.mj_grpo_profile_begin.argtypes = [C.c_int]

@@ -14,6 +14,7 @@
 
 #include "mj_grpo_kernels.hpp"
 #include "mj_norm_kernels.hpp"
+#include "mj_probe_kernels.hpp"
 
 namespace {
 
@@ -495,6 +496,20 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
                      size_t workspace_bytes, void* stream) {
   return run(kBackwardOnly, desc, hidden, lm_head, targets, old_logp, advantages, mask, nullptr, nullptr,
              nullptr, nullptr, lse, logp, d_hidden, d_lm_head, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"
+
+// ---- measurement support
+extern "C" {
+
+int mj_grpo_probe_mfma(const void* operands, float* out, int workgroups, int iters, double* flop, void* stream) {
+  if (!operands || !out) return fail(MJ_GRPO_ERR_NULL, "probe: operands/out is NULL");
+  if (workgroups <= 0 || workgroups > (1 << 16) || iters <= 0) return fail(MJ_GRPO_ERR_SHAPE, "probe: bad workgroups/iters");
+  if (misaligned(operands)) return fail(MJ_GRPO_ERR_ALIGN, "probe: operands must be 16-byte aligned");
+  mj::k_probe_mfma<<<workgroups, 256, 0, (hipStream_t)stream>>>((const mj::bf16x8*)operands, out, iters);
+  if (flop) *flop = (double)workgroups * 4.0 * iters * 2.0 * 16.0 * 32768.0;
+  return check_launch("k_probe_mfma");
 }
 
 }  // extern "C"
