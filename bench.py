@@ -181,6 +181,9 @@ def main() -> int:
                     help="instead of the loss: run the library's MFMA-only loop (no memory traffic) for ~3 s each with "
                          "random and with all-zero bf16 operands and print what the matrix cores sustain under the "
                          "power cap, with amd-smi power / clock samples")
+    ap.add_argument("--entropy-coef", type=float, default=0.0,
+                    help="add PPO's entropy bonus (plugins/training/ppo/module.py:140): times the running-maximum "
+                         "kernels + the in-place dZ pass instead of the default path")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-masked", action="store_true",
@@ -214,6 +217,7 @@ def main() -> int:
     cfg = M.CONFIGS[args.config]
     kw = dict(epsilon_low=cfg.eps_low, epsilon_high=cfg.eps_high, final_logit_softcap=cfg.softcap,
               chunk_tokens=args.chunk_tokens or None, dhidden_splits=args.dhidden_splits)
+    step_kw = dict(entropy_coef=args.entropy_coef) if args.entropy_coef else {}
 
     def logp_fn(wl):
         with torch.no_grad():
@@ -232,7 +236,7 @@ def main() -> int:
         return M.grpo_loss_value_and_grad(
             wl["hidden"], wl["lm_head"], wl["target_ids"], wl["old_logps"], wl["advantages"], wl["mask"],
             total_valid_token_count=wl["total_valid_token_count"], seq_shape=wl["seq_shape"],
-            return_token_entropy=cfg.token_entropy, skip_masked=skip_masked, **kw)
+            return_token_entropy=cfg.token_entropy, skip_masked=skip_masked, **step_kw, **kw)
 
     if args.zero_operands:
         wl["hidden"].zero_()
@@ -300,6 +304,8 @@ def main() -> int:
         line["smi"] = sampler.summary(t0, t_end)
     if args.zero_operands:
         line["config"]["operands"] = "all-zero hidden and lm_head"
+    if args.entropy_coef:
+        line["config"]["entropy_coef"] = args.entropy_coef
     line["config"]["skip_masked"] = bool(args.skip_masked)
     if not args.skip_masked and not args.no_skip_masked_extra:
         # Not the headline: the same step with tokens that cannot carry a gradient (mask 0, advantage 0)
