@@ -131,6 +131,44 @@ int mj_grpo_forward_backward(const MjGrpoDesc* desc, const void* hidden, const v
                              float* d_lm_head, void* workspace, size_t workspace_bytes,
                              void* stream);
 
+/* PPO actor-critic: the critic's value head and clipped value loss ride the same call
+ * (plugins/training/ppo/module.py:34-39, :52, :104-140).  All pointers are device pointers.
+ *   value_pred[t] = hidden[t, :] . value_w + value_b[0]                          (Dense(1), float32)
+ *   returns      NULL: advantages + value_pred, NOT detached (:107);   old_values NULL: stop_gradient(value_pred) (:118)
+ *   vl_t = use_clip ? max((v - R)^2, (old + clip(v - old, +-value_clip) - R)^2) : (v - R)^2       (:131-136)
+ *   value_loss[0] = sum(vl * mask) * inv_total_valid_tokens                                       (:138)
+ * The gradient of value_coef * value_loss reaches d_hidden inside the d_hidden product's epilogue
+ * (d_hidden[t, :] += dv_t * value_w), d_value_w[H] and d_value_b[1] are written in float32, all scaled by
+ * grad_loss_scale.  loss[0] stays policy loss - entropy_coef * entropy; the caller adds
+ * value_coef * value_loss[0] (:140).  value_w and d_value_w must be 16-byte aligned. */
+typedef struct MjPpoValue {
+  const float* value_w;      /* [H] */
+  const float* value_b;      /* [1] */
+  const float* returns;      /* [N] or NULL */
+  const float* old_values;   /* [N] or NULL */
+  float value_coef;          /* PPOActorCriticModule.value_coef */
+  float value_clip;          /* PPOActorCriticModule.value_clip_range when use_clip != 0 */
+  int32_t use_clip;          /* value_clip_range is not None */
+  int32_t reserved;
+  float* values;             /* out [N]: value_pred */
+  float* value_loss;         /* out [1] */
+  float* d_value_w;          /* out [H] */
+  float* d_value_b;          /* out [1] */
+} MjPpoValue;
+
+/* mj_grpo_forward_backward with the value head (value != NULL required).  The workspace size is
+ * that of mj_grpo_workspace_bytes plus mj_grpo_value_workspace_bytes, the extra part at the end. */
+int mj_grpo_value_workspace_bytes(const MjGrpoDesc* desc, size_t* extra_bytes);
+int mj_grpo_forward_backward_value(const MjGrpoDesc* desc, const MjPpoValue* value, const void* hidden,
+                                   const void* lm_head, const int32_t* targets, const float* old_logp,
+                                   const float* advantages, const float* mask, float* logp, float* lse,
+                                   float* token_entropy, float* loss, void* d_hidden, float* d_lm_head,
+                                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* The value head alone (PPOActorCriticModule.value, module.py:55-57): values[n] = hidden . value_w + value_b. */
+int mj_value_head_forward(const void* hidden, int64_t ld_hidden, const float* value_w, const float* value_b,
+                          float* values, int64_t n, int64_t h, void* stream);
+
 /* Backward from a saved forward (lse[N], logp[N]): recomputes the logits chunk by chunk
  * (8*N*H*V flop with the forward).  Same outputs as the backward half above.  For callers
  * that must separate the two passes (e.g. a forward under no-grad followed later by a

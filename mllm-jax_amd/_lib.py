@@ -16,7 +16,8 @@ FLAG_SFT = 1 << 1
 FLAG_SKIP_MASKED = 1 << 2
 
 EXPORTS = ("mj_grpo_version", "mj_grpo_last_error", "mj_grpo_workspace_bytes", "mj_grpo_forward",
-           "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_forward_noalloc", "mj_grpo_probe_mfma", "mj_grpo_profile_begin", "mj_grpo_profile_end",
+           "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_forward_noalloc", "mj_grpo_probe_mfma", "mj_grpo_forward_backward_value",
+           "mj_grpo_value_workspace_bytes", "mj_value_head_forward", "mj_grpo_profile_begin", "mj_grpo_profile_end",
            "mj_grpo_group_advantages", "mj_grpo_advantages", "mj_grpo_gae", "mj_rmsnorm_forward", "mj_sample_logits", "mj_sample_top_k", "mj_rmsnorm_workspace_bytes", "mj_rmsnorm_backward")
 
 KERNEL_NAMES = ("k_logits_stats", "k_finalize", "k_dz", "k_dhidden", "k_dhidden_reduce", "k_dw",
@@ -31,6 +32,14 @@ class MjGrpoDesc(C.Structure):
         ("softcap", C.c_float), ("inv_total_valid_tokens", C.c_float), ("grad_loss_scale", C.c_float),
         ("flags", C.c_uint32), ("dhidden_splits", C.c_uint32),
         ("entropy_coef", C.c_float), ("inv_entropy_count", C.c_float),
+    ]
+
+
+class MjPpoValue(C.Structure):
+    _fields_ = [
+        ("value_w", C.c_void_p), ("value_b", C.c_void_p), ("returns", C.c_void_p), ("old_values", C.c_void_p),
+        ("value_coef", C.c_float), ("value_clip", C.c_float), ("use_clip", C.c_int32), ("reserved", C.c_int32),
+        ("values", C.c_void_p), ("value_loss", C.c_void_p), ("d_value_w", C.c_void_p), ("d_value_b", C.c_void_p),
     ]
 
 
@@ -61,6 +70,10 @@ def load() -> C.CDLL:
     lib.mj_grpo_forward_noalloc.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp]
     lib.mj_grpo_probe_mfma.argtypes = [vp, fp, C.c_int, C.c_int, C.POINTER(C.c_double), vp]
     lib.mj_grpo_forward_backward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp, fp, vp, sz, vp]
+    lib.mj_grpo_forward_backward_value.argtypes = [dp, C.POINTER(MjPpoValue), vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp, fp,
+                                                   vp, sz, vp]
+    lib.mj_grpo_value_workspace_bytes.argtypes = [dp, C.POINTER(sz)]
+    lib.mj_value_head_forward.argtypes = [vp, C.c_int64, fp, fp, fp, C.c_int64, C.c_int64, vp]
     lib.mj_grpo_backward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, vp, fp, vp, sz, vp]
     lib.mj_grpo_profile_begin.argtypes = [C.c_int]
     lib.mj_grpo_profile_end.argtypes = [C.POINTER(C.c_double), C.POINTER(C.c_int)]
@@ -88,6 +101,12 @@ def workspace_bytes(desc: MjGrpoDesc) -> tuple[int, int]:
     f, b = C.c_size_t(0), C.c_size_t(0)
     check(load().mj_grpo_workspace_bytes(C.byref(desc), C.byref(f), C.byref(b)))
     return f.value, b.value
+
+
+def value_workspace_bytes(desc: MjGrpoDesc) -> int:
+    b = C.c_size_t(0)
+    check(load().mj_grpo_value_workspace_bytes(C.byref(desc), C.byref(b)))
+    return b.value
 
 
 def profile_begin(max_launches: int = 4096) -> None:

@@ -68,6 +68,8 @@ struct Plan {
   // token compaction (MJ_GRPO_FLAG_SKIP_MASKED): slot-order copies of the inputs and outputs
   bool compact;
   size_t perm, n_live, hid_p, tgt_p, fin_p[5], fout_p[3], dh_p;
+  // value head (mj_grpo_forward_backward_value): laid out behind total_bwd
+  size_t v_term, v_dv, v_dv_p, v_part, total_value;
 };
 
 // Splits of the dHidden product over the vocab: its (n/256) x (H/256) tiles rarely fill the 256
@@ -148,6 +150,11 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   p->zt = take((size_t)p->n_pad * p->ld_z * 2);
   p->part = take(p->dh_splits > 1 ? (size_t)p->dh_splits * p->n_pad * p->H * 4 : 0);
   p->total_bwd = o;
+  p->v_term = take((size_t)p->N * 4);
+  p->v_dv = take((size_t)rup(p->N, 256) * 4);
+  p->v_dv_p = take(p->compact ? (size_t)rup(p->N, 256) * 4 : 0);
+  p->v_part = take((size_t)((p->N + mj::kValueRows - 1) / mj::kValueRows) * p->H * 4);
+  p->total_value = o;
   return MJ_GRPO_OK;
 }
 
@@ -181,7 +188,7 @@ enum Mode { kForward, kForwardBackward, kBackwardOnly };
 int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head, const int32_t* targets,
         const float* old_logp, const float* adv, const float* mask, float* logp, float* lse,
         float* ent, float* loss, const float* saved_lse, const float* saved_logp, void* d_hidden,
-        float* d_w, void* workspace, size_t ws_bytes, void* stream_v) {
+        float* d_w, void* workspace, size_t ws_bytes, void* stream_v, const MjPpoValue* pv = nullptr) {
   Plan p;
   int rc = make_plan(d, &p);
   if (rc) return rc;
@@ -195,7 +202,17 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     return fail(MJ_GRPO_ERR_UNSUPPORTED, "the separate backward does not carry the entropy bonus (entropy_coef must be 0)");
   if (bwd && (!d_hidden || !d_w)) return fail(MJ_GRPO_ERR_NULL, "d_hidden/d_lm_head is NULL");
   if (!workspace) return fail(MJ_GRPO_ERR_WORKSPACE, "workspace is NULL");
-  const size_t need = bwd ? p.total_bwd : p.total_fwd;
+  if (pv != nullptr) {
+    if (mode != kForwardBackward) return fail(MJ_GRPO_ERR_UNSUPPORTED, "the value head needs the fused forward + backward pass");
+    if (!pv->value_w || !pv->value_b || !pv->values || !pv->value_loss || !pv->d_value_w || !pv->d_value_b)
+      return fail(MJ_GRPO_ERR_NULL, "value head: value_w/value_b/values/value_loss/d_value_w/d_value_b is NULL");
+    if (misaligned(pv->value_w) || misaligned(pv->d_value_w))
+      return fail(MJ_GRPO_ERR_ALIGN, "value head: value_w and d_value_w must be 16-byte aligned");
+    if (!adv) return fail(MJ_GRPO_ERR_NULL, "value head: advantages is NULL");
+    if (!isfinite(pv->value_coef) || (pv->use_clip && !(pv->value_clip >= 0.f)))
+      return fail(MJ_GRPO_ERR_UNSUPPORTED, "value head: value_coef must be finite and value_clip >= 0");
+  }
+  const size_t need = pv != nullptr ? p.total_value : (bwd ? p.total_bwd : p.total_fwd);
   if (ws_bytes < need) return fail(MJ_GRPO_ERR_WORKSPACE, "workspace too small: %zu < %zu bytes", ws_bytes, need);
   if (misaligned(hidden) || misaligned(lm_head) || misaligned(workspace) ||
       (bwd && (misaligned(d_hidden) || misaligned(d_w))))
@@ -240,6 +257,29 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     if ((rc = enable_lds(mj::k_dw<BM, BN>))) return rc;
   }
 
+  // Value head (PPO critic), on the caller's token order: value_pred, the clipped value loss and
+  // dv = d(value_coef * value_loss)/d value_pred; d_hidden picks dv up in the d_hidden product.
+  const float* dv = nullptr;
+  if (pv != nullptr) {
+    float* dvw = (float*)(ws + p.v_dv);
+    float* vterm = (float*)(ws + p.v_term);
+    float* vpart = (float*)(ws + p.v_part);
+    mj::k_value_head<<<(unsigned)((N + 3) / 4), 256, 0, st>>>((const uint16_t*)hidden, d->ld_hidden, N, H, pv->value_w,
+                                                              pv->value_b, pv->values);
+    mj::ValueLossArgs v;
+    v.values = pv->values; v.adv = adv; v.mask = mask; v.returns = pv->returns; v.old_values = pv->old_values;
+    v.n = N; v.inv_tv = d->inv_total_valid_tokens; v.coef = pv->value_coef; v.clip = pv->value_clip;
+    v.use_clip = pv->use_clip; v.gscale = gscale; v.vterm = vterm; v.dv = dvw;
+    mj::k_value_loss<<<(unsigned)((N + 255) / 256), 256, 0, st>>>(v);
+    mj::k_sum<<<1, 1024, 0, st>>>(vterm, N, pv->value_loss);
+    mj::k_sum<<<1, 1024, 0, st>>>(dvw, N, pv->d_value_b);
+    const int vblocks = (N + mj::kValueRows - 1) / mj::kValueRows;
+    mj::k_value_wgrad<<<vblocks, 256, 0, st>>>((const uint16_t*)hidden, d->ld_hidden, N, H, dvw, vpart);
+    mj::k_value_wgrad_reduce<<<(unsigned)((H + 255) / 256), 256, 0, st>>>(vpart, vblocks, H, pv->d_value_w);
+    if ((rc = check_launch("value head kernels"))) return rc;
+    dv = dvw;
+  }
+
   // Token compaction: tokens that cannot carry a gradient go behind the others; everything below
   // then works on slot-order copies and the backward kernels stop at the device-side count.
   const int* n_live = nullptr;
@@ -259,6 +299,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     ga.hid_p = (uint16_t*)(ws + p.hid_p); ga.tgt = targets; ga.tgt_p = (int32_t*)(ws + p.tgt_p);
     const float* fin[5] = {old_logp, adv, mask, saved_lse, saved_logp};
     for (int i = 0; i < 5; ++i) { ga.f_in[i] = fin[i]; ga.f_out[i] = (float*)(ws + p.fin_p[i]); }
+    ga.f_in[5] = dv; ga.f_out[5] = (float*)(ws + p.v_dv_p);
     mj::k_gather_tokens<<<N, 256, 0, st>>>(ga);
     if ((rc = check_launch("token compaction"))) return rc;
     hidden = ws + p.hid_p; ld_hid = H;
@@ -268,6 +309,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     mask = (const float*)(ws + p.fin_p[2]);
     if (saved_lse) saved_lse = (const float*)(ws + p.fin_p[3]);
     if (saved_logp) saved_logp = (const float*)(ws + p.fin_p[4]);
+    if (dv) dv = (const float*)(ws + p.v_dv_p);
     if (logp) logp = (float*)(ws + p.fout_p[0]);
     if (lse) lse = (float*)(ws + p.fout_p[1]);
     if (ent) ent = (float*)(ws + p.fout_p[2]);
@@ -367,6 +409,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       h.splits = p.dh_splits; h.k_per_split = (int)p.dh_k_per_split;
       h.dh = (uint16_t*)d_hidden + c0 * ld_dh; h.ld_dh = ld_dh;
       h.part = part; h.n_live = n_live; h.c0 = (int)c0; h.rs = rs; h.state = state;
+      h.dv = dv ? dv + c0 : nullptr; h.wv = pv ? pv->value_w : nullptr;
       const mj::TileMap mh((nc + BM - 1) / BM, (H + BN - 1) / BN, 0, 2, h.splits);
       {
         Timed t(MJ_GRPO_K_DHIDDEN, st);
@@ -376,7 +419,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
         const int64_t work = (int64_t)nc * (H / 4);
         Timed t(MJ_GRPO_K_DHIDDEN_REDUCE, st);
         mj::k_dhidden_reduce<<<(unsigned)((work + 255) / 256), 256, 0, st>>>(part, h.splits, nc, n_pad, H, h.dh,
-                                                                           h.ld_dh, rs, state);
+                                                                           h.ld_dh, rs, state, h.dv, h.wv);
       }
 
       mj::DwArgs w;
@@ -488,6 +531,36 @@ int mj_grpo_forward_backward(const MjGrpoDesc* desc, const void* hidden, const v
                              void* stream) {
   return run(kForwardBackward, desc, hidden, lm_head, targets, old_logp, advantages, mask, logp, lse,
              token_entropy, loss, nullptr, nullptr, d_hidden, d_lm_head, workspace, workspace_bytes, stream);
+}
+
+int mj_grpo_value_workspace_bytes(const MjGrpoDesc* desc, size_t* extra_bytes) {
+  Plan p;
+  int rc = make_plan(desc, &p);
+  if (rc) return rc;
+  if (extra_bytes) *extra_bytes = p.total_value - p.total_bwd;
+  return MJ_GRPO_OK;
+}
+
+int mj_grpo_forward_backward_value(const MjGrpoDesc* desc, const MjPpoValue* value, const void* hidden,
+                                   const void* lm_head, const int32_t* targets, const float* old_logp,
+                                   const float* advantages, const float* mask, float* logp, float* lse,
+                                   float* token_entropy, float* loss, void* d_hidden, float* d_lm_head,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+  if (value == nullptr) return fail(MJ_GRPO_ERR_NULL, "value is NULL (use mj_grpo_forward_backward)");
+  return run(kForwardBackward, desc, hidden, lm_head, targets, old_logp, advantages, mask, logp, lse, token_entropy,
+             loss, nullptr, nullptr, d_hidden, d_lm_head, workspace, workspace_bytes, stream, value);
+}
+
+int mj_value_head_forward(const void* hidden, int64_t ld_hidden, const float* value_w, const float* value_b,
+                          float* values, int64_t n, int64_t h, void* stream) {
+  if (!hidden || !value_w || !value_b || !values) return fail(MJ_GRPO_ERR_NULL, "value head: NULL pointer argument");
+  if (n <= 0 || h <= 0 || n > (1ll << 30) || h > (1 << 20) || ld_hidden < h)
+    return fail(MJ_GRPO_ERR_SHAPE, "value head: bad shape n=%lld h=%lld ld=%lld", (long long)n, (long long)h, (long long)ld_hidden);
+  if (h % 8 || ld_hidden % 8 || misaligned(hidden) || misaligned(value_w))
+    return fail(MJ_GRPO_ERR_ALIGN, "value head: h and ld_hidden must be multiples of 8, hidden and value_w 16-byte aligned");
+  mj::k_value_head<<<(unsigned)((n + 3) / 4), 256, 0, (hipStream_t)stream>>>((const uint16_t*)hidden, ld_hidden, (int)n,
+                                                                            (int)h, value_w, value_b, values);
+  return check_launch("k_value_head");
 }
 
 int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head, const int32_t* targets,

@@ -635,6 +635,7 @@ struct DhArgs {
   int c0;
   const float* rs;    // [n_pad] row scale, applied when state == 0
   const int* state;
+  const float *dv, *wv;   // value head (PPO critic): d_hidden[t, :] += dv[t] * wv[:]; both null = none
 };
 
 template <int BM, int BN>
@@ -662,20 +663,24 @@ __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
     const uint32_t ld2 = (uint32_t)p.ld_dh * 2;
     const __amdgpu_buffer_rsrc_t rs = make_rsrc_wave(p.dh + (int64_t)row0 * p.ld_dh, (int64_t)rows * ld2);
     const __amdgpu_buffer_rsrc_t srs = make_rsrc_wave(p.rs + row0, (int64_t)rows * 4);   // rows past n read 0
+    const __amdgpu_buffer_rsrc_t dvs = make_rsrc_wave(p.dv == nullptr ? nullptr : p.dv + row0, (int64_t)rows * 4);
 #pragma unroll
     for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         // the four consecutive token rows of this lane in the 8-row group q of block mi
-        f32x4 sc = {1.f, 1.f, 1.f, 1.f};
+        f32x4 sc = {1.f, 1.f, 1.f, 1.f}, dvr = {0.f, 0.f, 0.f, 0.f};
         if (scaled) sc = load_b128(srs, (uint32_t)(lhi * 16), (uint32_t)(mi * 32 + q * 8) * 4);
+        if (p.dv != nullptr) dvr = load_b128(dvs, (uint32_t)(lhi * 16), (uint32_t)(mi * 32 + q * 8) * 4);
 #pragma unroll
         for (int ni = 0; ni < G::NI; ++ni) {
           const int col = n0 + wn * G::WN + ni * 32 + l31;
           const uint32_t voff = col < p.H ? (uint32_t)(lhi * 4 * ld2 + col * 2) : kOob;
+          const float wvc = (p.dv != nullptr && col < p.H) ? p.wv[col] : 0.f;
 #pragma unroll
           for (int j = 0; j < 4; ++j)
-            store_b16(f32_to_bf16(g.acc[mi][ni][q * 4 + j] * sc[j]), rs, voff, (uint32_t)(mi * 32 + q * 8 + j) * ld2);
+            store_b16(f32_to_bf16(fmaf(dvr[j], wvc, g.acc[mi][ni][q * 4 + j] * sc[j])), rs, voff,
+                      (uint32_t)(mi * 32 + q * 8 + j) * ld2);
         }
       }
   } else {
@@ -695,11 +700,11 @@ __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
   }
 }
 
-// dh[row, :] = bf16(scale * sum over splits of part[s, row, :]), fixed order; scale = rs[row] when the
-// 16-bit matrix held E (state == 0), else 1.
+// dh[row, :] = bf16(scale * sum over splits of part[s, row, :] + dv[row] * wv[:]), fixed order;
+// scale = rs[row] when the 16-bit matrix held E (state == 0), else 1.
 __global__ __launch_bounds__(256) void k_dhidden_reduce(const float* part, int splits, int n, int n_pad, int H,
                                                         uint16_t* dh, int64_t ld_dh, const float* rs,
-                                                        const int* state) {
+                                                        const int* state, const float* dv, const float* wv) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;   // one thread = 4 columns
   const int h4 = H / 4;
   if (i >= (int64_t)n * h4) return;
@@ -707,6 +712,7 @@ __global__ __launch_bounds__(256) void k_dhidden_reduce(const float* part, int s
   f32x4 a = *(const f32x4*)(part + (int64_t)row * H + c);
   for (int s = 1; s < splits; ++s) a += *(const f32x4*)(part + ((int64_t)s * n_pad + row) * H + c);
   if (*state == 0) a *= rs[row];
+  if (dv != nullptr) a += dv[row] * *(const f32x4*)(wv + c);       // value head: + dv[t] * wv[:]
   uint16_t* o = dh + (int64_t)row * ld_dh + c;
   const uint32_t lo = f32_to_bf16(a[0]) | ((uint32_t)f32_to_bf16(a[1]) << 16);
   const uint32_t hi = f32_to_bf16(a[2]) | ((uint32_t)f32_to_bf16(a[3]) << 16);
@@ -783,6 +789,114 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
   }
 }
 
+// ----------------------------------------------------------------------------- value head (PPO critic)
+// plugins/training/ppo/module.py:34-39, :52 (Dense(1) on the final hidden states) and :104-138 (clipped
+// value loss).  values[t] = hidden[t, :] . wv + b: one wavefront per token row, fp32 accumulation.
+__global__ __launch_bounds__(256) void k_value_head(const uint16_t* hid, int64_t ld_hid, int n, int H, const float* wv,
+                                                    const float* bv, float* values) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= n) return;
+  const uint16_t* x = hid + (int64_t)row * ld_hid;
+  float acc = 0.f;
+  for (int c = lane * 8; c < H; c += 512) {
+    const u32x4 v = *(const u32x4*)(x + c);
+    const f32x4 w0 = *(const f32x4*)(wv + c), w1 = *(const f32x4*)(wv + c + 4);
+    acc = fmaf(__uint_as_float(v[0] << 16), w0[0], acc);
+    acc = fmaf(__uint_as_float(v[0] & 0xffff0000u), w0[1], acc);
+    acc = fmaf(__uint_as_float(v[1] << 16), w0[2], acc);
+    acc = fmaf(__uint_as_float(v[1] & 0xffff0000u), w0[3], acc);
+    acc = fmaf(__uint_as_float(v[2] << 16), w1[0], acc);
+    acc = fmaf(__uint_as_float(v[2] & 0xffff0000u), w1[1], acc);
+    acc = fmaf(__uint_as_float(v[3] << 16), w1[2], acc);
+    acc = fmaf(__uint_as_float(v[3] & 0xffff0000u), w1[3], acc);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+  if (lane == 0) values[row] = acc + bv[0];
+}
+
+struct ValueLossArgs {
+  const float *values, *adv, *mask;
+  const float *returns;      // or null: advantages + value_pred, NOT detached (module.py:107)
+  const float *old_values;   // or null: stop_gradient(value_pred) (:118)
+  int n;
+  float inv_tv, coef, clip, gscale;
+  int use_clip;              // value_clip_range is not None
+  float* vterm;              // [n] value_loss_t * mask_t / tvtc
+  float* dv;                 // [n] d(coef * value_loss)/d value_pred_t, times gscale
+};
+
+// Per token: max((v - R)^2, (old + clip(v - old, +-c) - R)^2) and its derivative with respect to
+// v (module.py:131-138).  Where the two arguments of the maximum are equal each gets half of the
+// cotangent (lax.max), which matters in the default case R = adv + v, old = v: both are adv^2.
+__global__ __launch_bounds__(256) void k_value_loss(ValueLossArgs p) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= p.n) return;
+  const float vp = p.values[t], mk = p.mask[t];
+  const bool rt_free = p.returns == nullptr;
+  const float rt = rt_free ? p.adv[t] + vp : p.returns[t];
+  const float ov = p.old_values == nullptr ? vp : p.old_values[t];
+  const float a = (vp - rt) * (vp - rt);
+  const float da = rt_free ? 0.f : 2.f * (vp - rt);
+  float vl = a, dvl = da;
+  if (p.use_clip) {
+    const float delta = vp - ov;
+    const float clipped = ov + fminf(fmaxf(delta, -p.clip), p.clip);
+    const float inside = fabsf(delta) <= p.clip ? 1.f : 0.f;
+    const float b = (clipped - rt) * (clipped - rt);
+    const float db = 2.f * (clipped - rt) * (inside - (rt_free ? 1.f : 0.f));
+    vl = fmaxf(a, b);
+    dvl = a > b ? da : (a < b ? db : 0.5f * (da + db));
+  }
+  p.vterm[t] = vl * mk * p.inv_tv;
+  p.dv[t] = p.coef * dvl * mk * p.inv_tv * p.gscale;
+}
+
+// out[0] = sum of x[0..n), one workgroup, fixed order
+__global__ __launch_bounds__(1024) void k_sum(const float* x, int n, float* out) {
+  __shared__ float sh[1024];
+  float a = 0.f;
+  for (int i = threadIdx.x; i < n; i += 1024) a += x[i];
+  sh[threadIdx.x] = a;
+  __syncthreads();
+  for (int o = 512; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) sh[threadIdx.x] += sh[threadIdx.x + o];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[0] = sh[0];
+}
+
+// d_wv[c] = sum_t dv[t] * hidden[t, c]: a workgroup adds up kValueRows rows (8 columns per thread,
+// rows in order), k_value_wgrad_reduce adds the workgroups' partial rows in fixed order.
+constexpr int kValueRows = 64;
+__global__ __launch_bounds__(256) void k_value_wgrad(const uint16_t* hid, int64_t ld_hid, int n, int H,
+                                                     const float* dv, float* part) {
+  const int r0 = blockIdx.x * kValueRows, r1 = min(r0 + kValueRows, n);
+  for (int c = threadIdx.x * 8; c < H; c += 2048) {
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int r = r0; r < r1; ++r) {
+      const float d = dv[r];
+      const u32x4 v = *(const u32x4*)(hid + (int64_t)r * ld_hid + c);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[2 * j] = fmaf(d, __uint_as_float(v[j] << 16), acc[2 * j]);
+        acc[2 * j + 1] = fmaf(d, __uint_as_float(v[j] & 0xffff0000u), acc[2 * j + 1]);
+      }
+    }
+    float* o = part + (int64_t)blockIdx.x * H + c;
+    *(f32x4*)o = f32x4{acc[0], acc[1], acc[2], acc[3]};
+    *(f32x4*)(o + 4) = f32x4{acc[4], acc[5], acc[6], acc[7]};
+  }
+}
+
+__global__ __launch_bounds__(256) void k_value_wgrad_reduce(const float* part, int blocks, int H, float* d_wv) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= H) return;
+  float a = 0.f;
+  for (int b = 0; b < blocks; ++b) a += part[(int64_t)b * H + c];
+  d_wv[c] = a;
+}
+
 // ----------------------------------------------------------------------------- compaction
 // Optional: tokens whose gradient is zero by construction (mask 0, or advantage 0 where nothing
 // else feeds the gradient) are moved behind the others so that the backward kernels can stop at
@@ -825,8 +939,8 @@ struct GatherArgs {
   const uint16_t* hid; int64_t ld_hid;     // [n, ld_hid] -> hid_p [n, H]
   uint16_t* hid_p;
   const int32_t* tgt; int32_t* tgt_p;
-  const float *f_in[5];                    // old_logp, adv, mask, saved_lse, saved_logp (any may be null)
-  float* f_out[5];
+  const float *f_in[6];                    // old_logp, adv, mask, saved_lse, saved_logp, dv (any may be null)
+  float* f_out[6];
 };
 
 // one workgroup per slot: copies the token's hidden row (16 bytes per thread and step) and scalars
@@ -836,7 +950,7 @@ __global__ __launch_bounds__(256) void k_gather_tokens(GatherArgs p) {
   u32x4* out = (u32x4*)(p.hid_p + (int64_t)j * p.H);
   for (int c = threadIdx.x; c < (p.H >> 3); c += 256) out[c] = in[c];
   if (threadIdx.x == 0) p.tgt_p[j] = p.tgt[src];
-  if (threadIdx.x < 5 && p.f_in[threadIdx.x] != nullptr) p.f_out[threadIdx.x][j] = p.f_in[threadIdx.x][src];
+  if (threadIdx.x < 6 && p.f_in[threadIdx.x] != nullptr) p.f_out[threadIdx.x][j] = p.f_in[threadIdx.x][src];
 }
 
 struct ScatterArgs {

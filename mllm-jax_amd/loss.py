@@ -143,8 +143,10 @@ class _Prepared:
                 _ptr(self.adv), _ptr(self.mask), _ptr(self.logp), _ptr(self.lse), _ptr(self.ent),
                 _ptr(self.loss), _ptr(ws), ws.numel(), self.stream()))
 
-    def forward_backward(self, d_w: Optional[torch.Tensor] = None):
+    def forward_backward(self, d_w: Optional[torch.Tensor] = None, value: Optional["_ValueHead"] = None):
         _, both = _lib.workspace_bytes(self.desc)
+        if value is not None:
+            both += _lib.value_workspace_bytes(self.desc)
         ws = _workspace(self.device, both)
         # d_hidden is written with the row pitch of hidden (the descriptor has one ld_hidden for both)
         ld = self.hidden.stride(0)
@@ -152,10 +154,17 @@ class _Prepared:
         if d_w is None:
             d_w = torch.empty((self.h, self.w.stride(0)), dtype=torch.float32, device=self.device)
         with torch.cuda.device(self.device):
-            _lib.check(_lib.load().mj_grpo_forward_backward(
-                C.byref(self.desc), _ptr(self.hidden), _ptr(self.w), _ptr(self.targets), _ptr(self.old),
-                _ptr(self.adv), _ptr(self.mask), _ptr(self.logp), _ptr(self.lse), _ptr(self.ent),
-                _ptr(self.loss), _ptr(d_h), _ptr(d_w), _ptr(ws), ws.numel(), self.stream()))
+            if value is None:
+                _lib.check(_lib.load().mj_grpo_forward_backward(
+                    C.byref(self.desc), _ptr(self.hidden), _ptr(self.w), _ptr(self.targets), _ptr(self.old),
+                    _ptr(self.adv), _ptr(self.mask), _ptr(self.logp), _ptr(self.lse), _ptr(self.ent),
+                    _ptr(self.loss), _ptr(d_h), _ptr(d_w), _ptr(ws), ws.numel(), self.stream()))
+            else:
+                _lib.check(_lib.load().mj_grpo_forward_backward_value(
+                    C.byref(self.desc), C.byref(value.struct(self.n, self.h, self.device)), _ptr(self.hidden),
+                    _ptr(self.w), _ptr(self.targets), _ptr(self.old), _ptr(self.adv), _ptr(self.mask),
+                    _ptr(self.logp), _ptr(self.lse), _ptr(self.ent), _ptr(self.loss), _ptr(d_h), _ptr(d_w),
+                    _ptr(ws), ws.numel(), self.stream()))
         return d_h, d_w[:, : self.v]
 
     def metrics(self, return_token_entropy: bool, sft: bool = False) -> dict:
@@ -180,6 +189,37 @@ class _Prepared:
         if self.desc.inv_entropy_count != 0.0:
             out["masked_mean_entropy"] = self.loss[1]
         return out
+
+
+class _ValueHead:
+    """Device arguments and outputs of the critic's value head for one fused call
+    (include/mj_grpo.h: MjPpoValue; plugins/training/ppo/module.py:34-39, :104-138)."""
+
+    def __init__(self, weight, bias, returns, old_values, value_coef, value_clip_range):
+        self.w = weight.detach().reshape(-1).to(torch.float32).contiguous()
+        self.b = bias.detach().reshape(-1)[:1].to(torch.float32).contiguous()
+        self.returns, self.old_values = returns, old_values
+        self.coef, self.clip = float(value_coef), value_clip_range
+        self.values = self.value_loss = self.d_w = self.d_b = None
+
+    def struct(self, n: int, h: int, device) -> "_lib.MjPpoValue":
+        if self.w.numel() != h:
+            raise ValueError(f"value head weight has {self.w.numel()} elements, expected hidden size {h}")
+        f32 = lambda x, name: None if x is None else _as_f32(x, n, device, name)
+        self.returns, self.old_values = f32(self.returns, "returns"), f32(self.old_values, "old_values")
+        self.values = torch.empty(n, dtype=torch.float32, device=device)
+        self.value_loss = torch.empty(1, dtype=torch.float32, device=device)
+        self.d_w = torch.empty(h, dtype=torch.float32, device=device)
+        self.d_b = torch.empty(1, dtype=torch.float32, device=device)
+        v = _lib.MjPpoValue()
+        v.value_w, v.value_b = self.w.data_ptr(), self.b.data_ptr()
+        v.returns, v.old_values = _ptr(self.returns), _ptr(self.old_values)
+        v.value_coef = self.coef
+        v.use_clip = 0 if self.clip is None else 1
+        v.value_clip = 0.0 if self.clip is None else float(self.clip)
+        v.values, v.value_loss = self.values.data_ptr(), self.value_loss.data_ptr()
+        v.d_value_w, v.d_value_b = self.d_w.data_ptr(), self.d_b.data_ptr()
+        return v
 
 
 _DEFAULTS = dict(total_valid_token_count=None, epsilon_low=0.2, epsilon_high=0.3, temperature=1.0,
@@ -265,30 +305,39 @@ def _poison_unless_one(grad_loss: torch.Tensor) -> torch.Tensor:
 
 
 class _FusedLossFn(torch.autograd.Function):
+    """loss = policy loss - entropy_coef * entropy [+ value_coef * value_loss] with the gradients the
+    kernels wrote in the same pass.  value_w / value_b / value are None without a value head."""
+
     @staticmethod
-    def forward(ctx, hidden, lm_head, prepared: _Prepared, want_grad: bool):
+    def forward(ctx, hidden, lm_head, prepared: _Prepared, want_grad: bool, value_w=None, value_b=None,
+                value: Optional[_ValueHead] = None):
         ctx.direct = ctx.terminal = False
-        ctx.d_w = ctx.buf = None
+        ctx.d_w = ctx.buf = ctx.value = None
         if want_grad:
             buf = _accumulate_target.buffer if lm_head.requires_grad else None
             if buf is not None:
                 _check_accumulator(buf, prepared)
                 prepared.desc.flags |= _lib.FLAG_DW_ACCUMULATE
-                d_h, _ = prepared.forward_backward(buf)
+                d_h, _ = prepared.forward_backward(buf, value)
                 _accumulate_target.uses += 1
                 ctx.direct, ctx.buf = True, buf
                 ctx.save_for_backward(d_h)
             elif _accumulate_target.terminal:
-                d_h, d_w = prepared.forward_backward()
+                d_h, d_w = prepared.forward_backward(None, value)
                 ctx.terminal, ctx.d_w = True, d_w      # kept out of save_for_backward: poisoned in place on misuse
                 ctx.save_for_backward(d_h)
             else:
-                d_h, d_w = prepared.forward_backward()
+                d_h, d_w = prepared.forward_backward(None, value)
                 ctx.save_for_backward(d_h, d_w)
             ctx.shapes = (hidden.shape, hidden.dtype, lm_head.dtype)
+            if value is not None:
+                ctx.value = (value.d_w, value.d_b, value_w.shape, value_w.dtype, value_b.shape, value_b.dtype)
         else:
             prepared.forward()
-        return prepared.loss[0].clone()
+        loss = prepared.loss[0].clone()
+        if value is not None and value.value_loss is not None:
+            loss = loss + value.coef * value.value_loss[0]
+        return loss
 
     @staticmethod
     def backward(ctx, grad_loss):
@@ -306,7 +355,12 @@ class _FusedLossFn(torch.autograd.Function):
             d_h, d_w = ctx.saved_tensors
             gw = (d_w * grad_loss).to(w_dtype)
         gh = (d_h * grad_loss.to(d_h.dtype)).reshape(shape).to(h_dtype)
-        return gh, gw, None, None
+        gwv = gbv = None
+        if ctx.value is not None:
+            d_wv, d_bv, wv_shape, wv_dtype, bv_shape, bv_dtype = ctx.value
+            gwv = (d_wv * grad_loss).reshape(wv_shape).to(wv_dtype)
+            gbv = (d_bv * grad_loss).reshape(bv_shape).to(bv_dtype)
+        return gh, gw, None, None, gwv, gbv, None
 
 
 def grpo_fused_loss(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
@@ -322,7 +376,7 @@ def grpo_fused_loss(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
     opts = {**_DEFAULTS, **kw}
     p = _Prepared(hidden, lm_head, target_ids, old_logps, advantages, mask, **opts)
     want = torch.is_grad_enabled() and (hidden.requires_grad or lm_head.requires_grad)
-    loss = _FusedLossFn.apply(hidden, lm_head, p, want)
+    loss = _FusedLossFn.apply(hidden, lm_head, p, want, None, None, None)
     out = p.metrics(return_token_entropy)
     out["loss"] = loss
     return out
@@ -338,7 +392,7 @@ def sft_fused_loss(hidden, lm_head, labels, valid, **kw) -> dict:
     safe = torch.where(validb, labels.reshape(-1), torch.zeros_like(labels.reshape(-1)))
     p = _Prepared(hidden, lm_head, safe, None, None, validb.to(torch.float32), sft=True, **opts)
     want = torch.is_grad_enabled() and (hidden.requires_grad or lm_head.requires_grad)
-    loss = _FusedLossFn.apply(hidden, lm_head, p, want)
+    loss = _FusedLossFn.apply(hidden, lm_head, p, want, None, None, None)
     out = p.metrics(False, sft=True)
     out["loss"] = loss
     return out
@@ -362,7 +416,8 @@ class TrainGRPOModule:
                  ref_model: Any = None, beta: float = 0.04, temperature: float = 1.0,
                  max_lengths: float = 2048, epsilon_low: float = 0.2, epsilon_high: float = 0.3,
                  entropy_threshold: float = 0.3, final_logit_softcap: Optional[float] = None,
-                 chunk_tokens: Optional[int] = None, skip_masked: bool = False):
+                 chunk_tokens: Optional[int] = None, skip_masked: bool = False, dhidden_splits: int = 0):
+        self.dhidden_splits = dhidden_splits
         self.model, self.lm_head = model, lm_head
         self.pad_token_id, self.num_pre_Q, self.ref_model, self.beta = pad_token_id, num_pre_Q, ref_model, beta
         self.temperature, self.max_lengths = temperature, max_lengths
@@ -385,7 +440,7 @@ class TrainGRPOModule:
             total_valid_token_count=inputs.get("total_valid_token_count"),
             epsilon_low=self.epsilon_low, epsilon_high=self.epsilon_high, temperature=self.temperature,
             final_logit_softcap=self.final_logit_softcap, seq_shape=(b, l - 1),
-            chunk_tokens=self.chunk_tokens, skip_masked=self.skip_masked)
+            chunk_tokens=self.chunk_tokens, skip_masked=self.skip_masked, dhidden_splits=self.dhidden_splits)
 
 
 class PPOActorCriticModule:
@@ -403,21 +458,36 @@ class PPOActorCriticModule:
                  epsilon_low: float = 0.2, epsilon_high: float = 0.2, value_coef: float = 0.5,
                  value_clip_range: Optional[float] = 0.2, entropy_coef: float = 0.0,
                  final_logit_softcap: Optional[float] = None, chunk_tokens: Optional[int] = None,
-                 skip_masked: bool = False):
-        self.skip_masked = skip_masked
+                 skip_masked: bool = False, dhidden_splits: int = 0):
+        self.skip_masked, self.dhidden_splits = skip_masked, dhidden_splits
         self.model, self.lm_head, self.value_head = model, lm_head, value_head
         self.temperature, self.epsilon_low, self.epsilon_high = temperature, epsilon_low, epsilon_high
         self.value_coef, self.value_clip_range, self.entropy_coef = value_coef, value_clip_range, entropy_coef
         self.final_logit_softcap, self.chunk_tokens = final_logit_softcap, chunk_tokens
 
+    def _head(self):
+        return self.value_head() if callable(self.value_head) else self.value_head
+
     def _values(self, hidden: torch.Tensor) -> torch.Tensor:
-        wv, bv = self.value_head() if callable(self.value_head) else self.value_head
-        # Dense(1), squeezed (module.py:52); accumulated and kept in float32 (the reference rounds
-        # the result to the activation dtype before casting it back to float32 at :127)
-        return (hidden.float() @ wv.reshape(-1, 1).float()).squeeze(-1) + bv.float()
+        """Dense(1), squeezed (module.py:52): one wavefront per token row, float32 accumulation and
+        result (the reference rounds the result to the activation dtype before casting it back to
+        float32 at :127)."""
+        wv, bv = self._head()
+        if hidden.device.type != "cuda":
+            raise RuntimeError("the value head needs tensors on an MI355X device; there is no CPU path")
+        shape = hidden.shape[:-1]
+        h2 = _Prepared._operand(hidden.detach().reshape(-1, hidden.shape[-1]).to(torch.bfloat16))
+        w = wv.detach().reshape(-1).to(torch.float32).contiguous()
+        b = bv.detach().reshape(-1)[:1].to(torch.float32).contiguous()
+        out = torch.empty(h2.shape[0], dtype=torch.float32, device=hidden.device)
+        with torch.cuda.device(hidden.device):
+            _lib.check(_lib.load().mj_value_head_forward(
+                h2.data_ptr(), h2.stride(0), w.data_ptr(), b.data_ptr(), out.data_ptr(), h2.shape[0], h2.shape[1],
+                torch.cuda.current_stream(hidden.device).cuda_stream))
+        return out.reshape(shape)
 
     def value(self, input_ids, attention_mask) -> torch.Tensor:
-        """module.py:55-57."""
+        """module.py:55-57 (no gradient: use __call__ for training)."""
         return self._values(self.model(input_ids=input_ids, attention_mask=attention_mask))
 
     @staticmethod
@@ -437,45 +507,56 @@ class PPOActorCriticModule:
         input_ids, labels = inputs["input_ids"], inputs["labels"]
         hidden = self.model(input_ids=input_ids, attention_mask=inputs["attention_mask"])
         w = self.lm_head() if callable(self.lm_head) else self.lm_head
+        wv, bv = self._head()
         b, l = input_ids.shape
         t = l - 1
         mask = labels[:, 1:].to(torch.float32)                                   # :67
-        value_pred = self._values(hidden)[:, :-1]                                # :104
-        advantages = self._like(inputs["advantages"], value_pred, "advantages")  # :87-94
+        advantages = self._like(inputs["advantages"], mask, "advantages")        # :87-94
         msum = mask.sum()
         tv = inputs.get("total_valid_token_count")
-        p = _Prepared(hidden[:, :-1, :].reshape(b * t, -1), w, input_ids[:, 1:].reshape(-1),
+        hid = hidden[:, :-1, :].reshape(b * t, -1)
+        p = _Prepared(hid, w, input_ids[:, 1:].reshape(-1),
                       inputs.get("old_per_token_logps"), advantages.reshape(-1), mask.reshape(-1),
                       total_valid_token_count=float(tv) if tv is not None else float(msum.item()),
                       epsilon_low=self.epsilon_low, epsilon_high=self.epsilon_high,
                       temperature=self.temperature, final_logit_softcap=self.final_logit_softcap,
                       seq_shape=(b, t), chunk_tokens=self.chunk_tokens, skip_masked=self.skip_masked,
-                      entropy_coef=self.entropy_coef,
+                      dhidden_splits=self.dhidden_splits, entropy_coef=self.entropy_coef,
                       entropy_token_count=float(msum.item()) if self.entropy_coef != 0.0 or tv is None else None)
-        want = torch.is_grad_enabled() and (hidden.requires_grad or w.requires_grad)
-        fused = _FusedLossFn.apply(hidden[:, :-1, :].reshape(b * t, -1), w, p, want)   # policy - coef * entropy
-        entropy = (p.ent.reshape(b, t) * mask).sum() / (msum + 1e-8)             # :77
-        policy_loss = (fused + self.entropy_coef * entropy).detach()
-
-        returns = inputs.get("returns")
-        if returns is None:
-            returns = advantages + value_pred                                    # :107 (not detached)
-        returns = self._like(returns, value_pred, "returns")
-        old_values = inputs.get("old_values", inputs.get("values"))
-        if old_values is None:
-            old_values = value_pred.detach()                                     # :118
-        old_values = self._like(old_values, value_pred, "old_values")
-        vp, rt, ov = value_pred.float(), returns.float(), old_values.float()
-        if self.value_clip_range is not None:
-            c = float(self.value_clip_range)
-            clipped = ov + torch.clamp(vp - ov, -c, c)
-            value_loss = torch.maximum((vp - rt) ** 2, (clipped - rt) ** 2)      # :133-134
+        returns = inputs.get("returns")                                          # :105-114
+        if returns is not None:
+            returns = self._like(returns, mask, "returns").to(torch.float32)
+        old_values = inputs.get("old_values", inputs.get("values"))              # :116-125
+        if old_values is not None:
+            old_values = self._like(old_values, mask, "old_values").to(torch.float32)
+        want = torch.is_grad_enabled() and (hidden.requires_grad or w.requires_grad or wv.requires_grad
+                                            or bv.requires_grad)
+        if want:
+            # value head, clipped value loss and their gradients inside the fused pass
+            head = _ValueHead(wv, bv, None if returns is None else returns.reshape(-1),
+                              None if old_values is None else old_values.reshape(-1), self.value_coef,
+                              self.value_clip_range)
+            loss = _FusedLossFn.apply(hid, w, p, True, wv, bv, head)             # :140
+            value_pred = head.values.reshape(b, t)
+            value_loss = head.value_loss[0]
         else:
-            value_loss = (vp - rt) ** 2
-        value_loss = (value_loss * mask).sum() / p.tv                            # :138
-        loss = fused + float(self.value_coef) * value_loss                       # :140
-        return {"loss": loss, "policy_loss": policy_loss, "value_loss": value_loss, "entropy": entropy,
-                "value_pred_mean": vp.mean(), "return_mean": rt.mean(),
+            fused = _FusedLossFn.apply(hid, w, p, False, None, None, None)
+            value_pred = self._values(hidden)[:, :-1]                            # :104
+            rt = advantages + value_pred if returns is None else returns
+            ov = value_pred if old_values is None else old_values
+            if self.value_clip_range is not None:
+                c = float(self.value_clip_range)
+                clipped = ov + torch.clamp(value_pred - ov, -c, c)
+                vl = torch.maximum((value_pred - rt) ** 2, (clipped - rt) ** 2)  # :133-134
+            else:
+                vl = (value_pred - rt) ** 2
+            value_loss = (vl * mask).sum() / p.tv                                # :138
+            loss = fused + float(self.value_coef) * value_loss
+        entropy = p.loss[1] if p.desc.inv_entropy_count != 0.0 else (p.ent.reshape(b, t) * mask).sum() / (msum + 1e-8)  # :77
+        policy_loss = (p.loss[0] + self.entropy_coef * entropy).detach()
+        rt_mean = (advantages + value_pred).mean() if returns is None else returns.mean()
+        return {"loss": loss, "policy_loss": policy_loss, "value_loss": value_loss.detach(), "entropy": entropy,
+                "value_pred_mean": value_pred.mean(), "return_mean": rt_mean,
                 "per_token_logps": p.logp.reshape(b, t)}
 
 

@@ -31,7 +31,7 @@ def _desc(lib, **kw):
 def test_header_symbols_are_exported(lib):
     header = open(os.path.join(ROOT, "include", "mj_grpo.h")).read() + open(os.path.join(ROOT, "include", "mj_norm.h")).read() \
         + open(os.path.join(ROOT, "include", "mj_sample.h")).read()
-    declared = set(re.findall(r"\b(mj_(?:grpo|rmsnorm|sample)_[a-z_]+)\s*\(", header))
+    declared = set(re.findall(r"\b(mj_(?:grpo|rmsnorm|sample|value)_[a-z_]+)\s*\(", header))
     assert declared == set(lib.EXPORTS)
     handle = lib.load()
     for name in declared:

@@ -78,6 +78,8 @@ def _run_case(seed, b, l, h, v, *, old_noise=0.0, returns=False, old_values=Fals
     out["loss"].backward()
     torch.cuda.synchronize()
 
+    for k in ("skip_masked", "dhidden_splits"):
+        hyper.pop(k, None)
     ohyper = {k: hyper[k] for k in ("epsilon_low", "epsilon_high", "value_coef", "value_clip_range",
                                     "entropy_coef", "final_logit_softcap") if k in hyper}
     ref = O.ppo_actor_critic_loss(hid_flat, w.float().numpy(), wv.numpy(), float(bv), y, old, adv_flat, mask,
@@ -122,6 +124,46 @@ def test_no_value_clip_and_per_sequence_advantages():
 def test_softcap_with_entropy_bonus_across_chunks():
     _run_case(7, 5, 129, 64, 1544, returns=True, old_values=True, entropy_coef=0.05, final_logit_softcap=5.0,
               chunk_tokens=256, old_noise=0.1)
+
+
+@pytest.mark.parametrize("splits", [1, 4])
+def test_value_head_gradient_joins_d_hidden_in_the_product(splits):
+    """entropy_coef = 0: the E-based backward; dv * value_w is added in the d_hidden product's own
+    epilogue (one split) or in the fixed-order sum of the split partials."""
+    _run_case(8, 4, 65, 136, 1000, returns=True, old_values=True, old_noise=0.1, value_coef=0.7,
+              dhidden_splits=splits)
+
+
+def test_value_head_with_skip_masked_and_chunks():
+    _run_case(9, 6, 97, 64, 776, returns=True, old_values=True, old_noise=0.1, chunk_tokens=256, skip_masked=True)
+    _run_case(10, 3, 41, 64, 520, skip_masked=True, entropy_coef=0.02, returns=True)
+
+
+def test_value_method_and_no_grad_call_match_the_oracle():
+    import mllm_jax_amd as M
+    dev = torch.device("cuda:0")
+    b, l, h, v = 3, 33, 72, 520
+    ids, emb, pos, w, wv, bv, labels, adv = _batch(12, b, l, h, v)
+    hidden = (emb[ids].float() + pos[None].float()).to(torch.bfloat16)
+    module = M.PPOActorCriticModule(lambda input_ids, attention_mask: hidden.to(dev), w.to(dev), (wv.to(dev), bv.to(dev)))
+    vals = module.value(ids.to(dev), torch.ones(b, l, device=dev))
+    ref_v = hidden.double().numpy() @ wv.double().numpy() + float(bv)
+    assert tuple(vals.shape) == (b, l) and vals.dtype == torch.float32
+    np.testing.assert_allclose(vals.cpu().numpy(), ref_v, atol=1e-4, rtol=1e-5)
+    t = l - 1
+    g = torch.Generator().manual_seed(13)
+    r = torch.from_numpy(ref_v[:, :-1]).float() + torch.randn(b, t, generator=g)
+    inputs = {"input_ids": ids.to(dev), "attention_mask": torch.ones(b, l, device=dev), "labels": labels.to(dev),
+              "advantages": adv.to(dev), "returns": r.to(dev)}
+    with torch.no_grad():
+        out = module(inputs)
+    ref = O.ppo_actor_critic_loss(hidden[:, :-1].reshape(b * t, h).float().numpy(), w.float().numpy(), wv.numpy(),
+                                  float(bv), ids[:, 1:].reshape(-1).numpy(), None, adv.reshape(-1).numpy(),
+                                  labels[:, 1:].reshape(-1).float().numpy(), returns=r.reshape(-1).numpy(),
+                                  with_grads=False)
+    for k in ("loss", "policy_loss", "value_loss", "entropy", "value_pred_mean", "return_mean"):
+        assert abs(float(out[k]) - ref[k]) <= LOSS_RTOL * abs(ref[k]) + 2e-6, k
+    assert not out["loss"].requires_grad
 
 
 def test_entropy_only_gradient_through_value_and_grad():
