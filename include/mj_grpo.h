@@ -180,7 +180,8 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
 
 /* Sequence-level advantage estimators on the device (host NumPy in the reference, evaluated by the
  * runner at runner/grpo_gsm8k.py:680).  rewards, advantages: float32 [b]; group_ids: int32 [b] (any
- * ids, any group sizes; unused by MJ_GRPO_ADV_GLOBAL).  b <= 65536.
+ * ids, any group sizes; unused by MJ_GRPO_ADV_GLOBAL).  b <= 65536 (MJ_GRPO_ADV_GLOBAL), b <= 8192 for the
+ * grouped estimators, which walk the batch once per sample.
  *   MJ_GRPO_ADV_GRPO    (r - mean_g) / (std_g + eps), population std     advantage/grpo.py:8-52
  *   MJ_GRPO_ADV_GLOBAL  (r - mean) / (std + eps)                          advantage/estimators.py:37-55
  *   MJ_GRPO_ADV_RLOO    r - mean of the others in the group (group mean for singletons); whiten != 0

@@ -662,6 +662,9 @@ int mj_grpo_advantages(int mode, const float* rewards, const int32_t* group_ids,
   if (!rewards || !advantages || (mode != mj::kAdvGlobal && !group_ids))
     return fail(MJ_GRPO_ERR_NULL, "rewards/group_ids/advantages is NULL");
   if (b <= 0 || b > (1 << 16)) return fail(MJ_GRPO_ERR_SHAPE, "batch must be in [1, 65536] (got %lld)", (long long)b);
+  // the grouped estimators walk the batch once per sample (a batch is hundreds of sequences)
+  if (mode != mj::kAdvGlobal && b > (1 << 13))
+    return fail(MJ_GRPO_ERR_SHAPE, "grouped advantage estimators take at most 8192 sequences (got %lld)", (long long)b);
   if (!(eps > 0.f)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "eps must be > 0");
   if (mode == mj::kAdvDapo && !(alpha >= 0.f)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "alpha must be >= 0");
   mj::AdvArgs a;

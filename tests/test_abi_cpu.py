@@ -193,3 +193,9 @@ int main(void) {
     run = subprocess.run([str(exe)], capture_output=True, text=True)
     assert run.returncode == 0, (run.returncode, run.stdout, run.stderr)
     assert "sizeof(MjGrpoDesc)=88" in run.stdout
+
+
+def test_grouped_advantage_estimators_cap_the_batch(lib):
+    handle = lib.load()
+    rc = handle.mj_grpo_advantages(0, 1, 1, 1, 8193, 1e-4, 0.0, 0, 0.0, None)   # pointers are never touched
+    assert rc == 2 and b"8192" in handle.mj_grpo_last_error()
