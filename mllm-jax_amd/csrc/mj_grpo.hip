@@ -327,7 +327,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     a.pm = pm; a.pl = pl; a.ps = ps; a.plt = plt; a.inv_t = inv_t; a.ld_p = p.n_pad;
     a.targets = targets + c0; a.zy = zy + c0; a.n_live = n_live; a.c0 = (int)c0;
     a.mask = mask + c0; a.lse = nullptr; a.g = g; a.state = state;
-    const mj::TileMap map((V + BM - 1) / BM, (nc + BN - 1) / BN, 1);
+    const mj::TileMap map = mj::TileMap::pick_shape((V + BM - 1) / BM, (nc + BN - 1) / BN, 1, 1);
 
     mj::FinalizeArgs f;
     f.pm = pm; f.pl = pl; f.ps = ps; f.plt = plt; f.inv_t = inv_t; f.ld_p = p.n_pad; f.parts = (int)p.parts;
@@ -410,7 +410,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       h.dh = (uint16_t*)d_hidden + c0 * ld_dh; h.ld_dh = ld_dh;
       h.part = part; h.n_live = n_live; h.c0 = (int)c0; h.rs = rs; h.state = state;
       h.dv = dv ? dv + c0 : nullptr; h.wv = pv ? pv->value_w : nullptr;
-      const mj::TileMap mh((nc + BM - 1) / BM, (H + BN - 1) / BN, 0, 2, h.splits);
+      const mj::TileMap mh = mj::TileMap::pick_shape((nc + BM - 1) / BM, (H + BN - 1) / BN, 0, h.splits);
       {
         Timed t(MJ_GRPO_K_DHIDDEN, st);
         mj::k_dhidden<BM, BN><<<mh.items(), mj::kThreads, lds, st>>>(h, mh);
@@ -427,7 +427,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       w.H = H; w.V = V; w.n = nc;
       w.dw = d_w; w.ld_dw = d->ld_w; w.n_live = n_live; w.c0 = (int)c0; w.state = state;
       w.accumulate = (c0 > 0 || (d->flags & MJ_GRPO_FLAG_DW_ACCUMULATE)) ? 1 : 0;
-      const mj::TileMap mw((V + BM - 1) / BM, (H + BN - 1) / BN, 0);
+      const mj::TileMap mw = mj::TileMap::pick_shape((V + BM - 1) / BM, (H + BN - 1) / BN, 0, 1);
       {
         Timed t(MJ_GRPO_K_DW, st);
         mj::k_dw<BM, BN><<<mw.items(), mj::kThreads, lds, st>>>(w, mw);
@@ -717,7 +717,7 @@ int mj_sample_logits(const void* hidden, int64_t ld_hidden, const void* lm_head,
   mj::LogitsRowsArgs a;
   a.w = (const __bf16*)lm_head; a.hid = (const __bf16*)hidden; a.ld_w = ld_w; a.ld_hid = ld_hidden;
   a.V = (int)vocab; a.n = (int)b; a.H = (int)h; a.cap = softcap; a.out = logits; a.ld_out = ld_logits;
-  const mj::TileMap map((int)((vocab + BM - 1) / BM), (int)((b + BN - 1) / BN), 1);
+  const mj::TileMap map = mj::TileMap::pick_shape((int)((vocab + BM - 1) / BM), (int)((b + BN - 1) / BN), 1, 1);
   mj::k_logits_rows<BM, BN><<<map.items(), mj::kThreads, mj::GemmTN<BM, BN>::kLdsBytes, (hipStream_t)stream>>>(a, map);
   return check_launch("k_logits_rows");
 }

@@ -644,7 +644,7 @@ __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   // Only token tiles that hold live tokens are walked: the tile list is rebuilt for that many
   // rows of tiles, so that the live work spreads evenly over the XCDs (ids past its end leave).
-  const TileMap live(live_pad(p.n_live, p.c0, p.n_pad) / BM, map.tiles_n, map.n_first, map.lgm, map.splits);
+  const TileMap live(live_pad(p.n_live, p.c0, p.n_pad) / BM, map.tiles_n, map.n_first, map.lgm, map.splits, map.lgs);
   int tm, tn, split;
   if (!live.tile(blockIdx.x, tm, tn, split)) return;
   const int m0 = tm * BM, n0 = tn * BN;
