@@ -184,6 +184,10 @@ def main() -> int:
     ap.add_argument("--entropy-coef", type=float, default=0.0,
                     help="add PPO's entropy bonus (plugins/training/ppo/module.py:140): times the running-maximum "
                          "kernels + the in-place dZ pass instead of the default path")
+    ap.add_argument("--no-kernel-events", action="store_true",
+                    help="time the steps without the per-kernel HIP events (each event pair leaves ~10 us between "
+                         "two kernels: nothing at the headline shape, 10 %% of a step at the smallest); the per-kernel "
+                         "figures and the roofline object then come from a second, short, instrumented loop")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--skip-masked", action="store_true",
@@ -250,7 +254,8 @@ def main() -> int:
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    _lib.profile_begin(64 * max(args.steps, 1))
+    if not args.no_kernel_events:
+        _lib.profile_begin(64 * max(args.steps, 1))
     sampler = _SmiSampler() if args.smi else None
     if sampler:
         sampler.__enter__()
@@ -264,6 +269,13 @@ def main() -> int:
     dt = t_end - t0
     if sampler:
         sampler.__exit__()
+    prof_steps = args.steps
+    if args.no_kernel_events:
+        prof_steps = min(args.steps, 5)
+        _lib.profile_begin(64 * prof_steps)
+        for _ in range(prof_steps):
+            step()
+        torch.cuda.synchronize()
     prof = _lib.profile_end()
 
     ms_per_step = dt / args.steps * 1e3
@@ -274,7 +286,7 @@ def main() -> int:
     gemms = {k: prof[k] for k in ("k_logits_stats", "k_dhidden", "k_dw")}
     dom = max(gemms, key=lambda k: gemms[k][0])
     dom_ms, dom_launches = gemms[dom]
-    flop_per_launch = 2.0 * n * h * v * args.steps / max(dom_launches, 1)   # algorithmic 2*n_chunk*H*V
+    flop_per_launch = 2.0 * n * h * v * prof_steps / max(dom_launches, 1)   # algorithmic 2*n_chunk*H*V
     avg_launch_ms = dom_ms / max(dom_launches, 1)
     achieved = flop_per_launch / (avg_launch_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
@@ -297,13 +309,15 @@ def main() -> int:
         "algorithmic_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 1),
         "loss": float(metrics["loss"].item()),
         "roofline": roofline,
-        "kernel_ms_per_step": {k: round(v_[0] / args.steps, 3) for k, v_ in prof.items()},
+        "kernel_ms_per_step": {k: round(v_[0] / prof_steps, 3) for k, v_ in prof.items()},
     }
 
     if sampler:
         line["smi"] = sampler.summary(t0, t_end)
     if args.zero_operands:
         line["config"]["operands"] = "all-zero hidden and lm_head"
+    if args.no_kernel_events:
+        line["config"]["kernel_events"] = "separate loop of %d steps after the timed one" % prof_steps
     if args.entropy_coef:
         line["config"]["entropy_coef"] = args.entropy_coef
     line["config"]["skip_masked"] = bool(args.skip_masked)

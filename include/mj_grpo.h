@@ -131,6 +131,14 @@ int mj_grpo_forward_backward(const MjGrpoDesc* desc, const void* hidden, const v
                              float* d_lm_head, void* workspace, size_t workspace_bytes,
                              void* stream);
 
+/* The two per-sequence entropy entries of the reference's return dict
+ * (MLLM_JAX/train_modules/__init__.py:141-157) from the per-token entropies of a forward:
+ * token_entropy, mask: float32 [b, t] row-major; entropy[b] = sum(H * mask) / sum(mask) (nan for an
+ * empty row, as in the reference); entropy_loss[b] = the mean of H over the tokens with mask == 1
+ * whose running count of such tokens lies in [4, 100]. */
+int mj_grpo_sequence_entropy(const float* token_entropy, const float* mask, int64_t b, int64_t t,
+                             float* entropy, float* entropy_loss, void* stream);
+
 /* PPO actor-critic: the critic's value head and clipped value loss ride the same call
  * (plugins/training/ppo/module.py:34-39, :52, :104-140).  All pointers are device pointers.
  *   value_pred[t] = hidden[t, :] . value_w + value_b[0]                          (Dense(1), float32)

@@ -17,7 +17,7 @@ FLAG_SKIP_MASKED = 1 << 2
 
 EXPORTS = ("mj_grpo_version", "mj_grpo_last_error", "mj_grpo_workspace_bytes", "mj_grpo_forward",
            "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_forward_noalloc", "mj_grpo_probe_mfma", "mj_grpo_forward_backward_value",
-           "mj_grpo_value_workspace_bytes", "mj_value_head_forward", "mj_grpo_profile_begin", "mj_grpo_profile_end",
+           "mj_grpo_value_workspace_bytes", "mj_value_head_forward", "mj_grpo_sequence_entropy", "mj_grpo_profile_begin", "mj_grpo_profile_end",
            "mj_grpo_group_advantages", "mj_grpo_advantages", "mj_grpo_gae", "mj_rmsnorm_forward", "mj_sample_logits", "mj_sample_top_k", "mj_rmsnorm_workspace_bytes", "mj_rmsnorm_backward")
 
 KERNEL_NAMES = ("k_logits_stats", "k_finalize", "k_dz", "k_dhidden", "k_dhidden_reduce", "k_dw",
@@ -74,6 +74,7 @@ def load() -> C.CDLL:
                                                    vp, sz, vp]
     lib.mj_grpo_value_workspace_bytes.argtypes = [dp, C.POINTER(sz)]
     lib.mj_value_head_forward.argtypes = [vp, C.c_int64, fp, fp, fp, C.c_int64, C.c_int64, vp]
+    lib.mj_grpo_sequence_entropy.argtypes = [fp, fp, C.c_int64, C.c_int64, fp, fp, vp]
     lib.mj_grpo_backward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, vp, fp, vp, sz, vp]
     lib.mj_grpo_profile_begin.argtypes = [C.c_int]
     lib.mj_grpo_profile_end.argtypes = [C.POINTER(C.c_double), C.POINTER(C.c_int)]

@@ -372,7 +372,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       }
       {
         Timed t(MJ_GRPO_K_FINALIZE, st);
-        mj::k_finalize<mj::kStatsExp><<<n_pad / 64, 64 * mj::kFinSlices, 0, st>>>(f);
+        mj::k_finalize<mj::kStatsExp><<<n_pad / mj::kFinTokens, mj::kFinTokens * mj::kFinSlices, 0, st>>>(f);
       }
       if (bwd) {
         const int64_t work = (int64_t)nc * (H / 8);
@@ -384,7 +384,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       Timed t(MJ_GRPO_K_RESCUE, st);
       f.rescue = 1; z.rescue = 1;
       mj::k_logits_stats<BM, BN, mj::kStatsMax, true><<<kRescueGrid, mj::kThreads, lds, st>>>(a, map);
-      mj::k_finalize<mj::kStatsMax><<<n_pad / 64, 64 * mj::kFinSlices, 0, st>>>(f);
+      mj::k_finalize<mj::kStatsMax><<<n_pad / mj::kFinTokens, mj::kFinTokens * mj::kFinSlices, 0, st>>>(f);
       if (bwd) mj::k_dz<<<dz_grid, 256, 0, st>>>(z);
     } else {
       {
@@ -393,7 +393,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       }
       {
         Timed t(MJ_GRPO_K_FINALIZE, st);
-        mj::k_finalize<mj::kStatsMax><<<n_pad / 64, 64 * mj::kFinSlices, 0, st>>>(f);
+        mj::k_finalize<mj::kStatsMax><<<n_pad / mj::kFinTokens, mj::kFinTokens * mj::kFinSlices, 0, st>>>(f);
       }
       if (bwd) {
         Timed t(MJ_GRPO_K_DZ, st);
@@ -531,6 +531,14 @@ int mj_grpo_forward_backward(const MjGrpoDesc* desc, const void* hidden, const v
                              void* stream) {
   return run(kForwardBackward, desc, hidden, lm_head, targets, old_logp, advantages, mask, logp, lse,
              token_entropy, loss, nullptr, nullptr, d_hidden, d_lm_head, workspace, workspace_bytes, stream);
+}
+
+int mj_grpo_sequence_entropy(const float* token_entropy, const float* mask, int64_t b, int64_t t, float* entropy,
+                             float* entropy_loss, void* stream) {
+  if (!token_entropy || !mask || !entropy || !entropy_loss) return fail(MJ_GRPO_ERR_NULL, "sequence_entropy: NULL pointer argument");
+  if (b <= 0 || t <= 0 || b > (1 << 24) || t > (1 << 24)) return fail(MJ_GRPO_ERR_SHAPE, "sequence_entropy: bad shape b=%lld t=%lld", (long long)b, (long long)t);
+  mj::k_sequence_entropy<<<(unsigned)((b + 3) / 4), 256, 0, (hipStream_t)stream>>>(token_entropy, mask, (int)b, (int)t, entropy, entropy_loss);
+  return check_launch("k_sequence_entropy");
 }
 
 int mj_grpo_value_workspace_bytes(const MjGrpoDesc* desc, size_t* extra_bytes) {

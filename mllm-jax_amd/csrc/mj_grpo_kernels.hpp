@@ -377,11 +377,12 @@ struct FinalizeArgs {
   int rescue;                  // kStatsMax launched behind a kStatsExp pass: leave unless state != 0
 };
 
-// block = (64 tokens) x (kFinSlices slices of the partial list)
-constexpr int kFinSlices = 16;
+// block = (kFinTokens tokens) x (kFinSlices slices of the partial list): few tokens per block keep a
+// small chunk spread over many CUs (a 512-token chunk walks 1188 partials per token)
+constexpr int kFinTokens = 16, kFinSlices = 64;
 template <int MODE>
-__global__ __launch_bounds__(64 * kFinSlices) void k_finalize(FinalizeArgs p) {
-  __shared__ float sm[kFinSlices][64], sl[kFinSlices][64], ss[kFinSlices][64], st[kFinSlices][64];
+__global__ __launch_bounds__(kFinTokens * kFinSlices) void k_finalize(FinalizeArgs p) {
+  __shared__ float sm[kFinSlices][kFinTokens], sl[kFinSlices][kFinTokens], ss[kFinSlices][kFinTokens], st[kFinSlices][kFinTokens];
   if (MODE == kStatsMax) {
     if (p.rescue) {
       if (__builtin_amdgcn_readfirstlane(*p.state) == 0) return;
@@ -389,8 +390,8 @@ __global__ __launch_bounds__(64 * kFinSlices) void k_finalize(FinalizeArgs p) {
       *p.state = 1;            // the 16-bit matrix of this chunk will hold dZ itself
     }
   }
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-  const int t = blockIdx.x * 64 + tx;
+  const int tx = threadIdx.x % kFinTokens, ty = threadIdx.x / kFinTokens;
+  const int t = blockIdx.x * kFinTokens + tx;
   const bool tempered = p.inv_t != 1.f;   // then s and lt are sums under softmax(z / T)
   float m = kNegBig, l = 0.f, s = 0.f, lt = 0.f;
   if (t < p.n) {
@@ -786,6 +787,54 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
           store_b128(c + a[mi][q], rs, voff, (uint32_t)vv * 4);
         }
     }
+  }
+}
+
+// ----------------------------------------------------------------------------- per-sequence entropy
+// MLLM_JAX/train_modules/__init__.py:141-157 on [b, t] row-major data, one wavefront per sequence:
+//   entropy[s]      = sum_t(H * mask) / sum_t(mask)                      (nan for an empty row, as there)
+//   entropy_loss[s] = the same mean over the window  mask == 1  and  4 <= cumsum(mask == 1) <= 100
+// Lane l owns the l-th contiguous piece of the row, so the running count of valid tokens is a prefix
+// sum over lanes.
+__global__ __launch_bounds__(256) void k_sequence_entropy(const float* ent, const float* mask, int b, int t,
+                                                          float* entropy, float* entropy_loss) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= b) return;
+  const float* e = ent + (int64_t)row * t;
+  const float* m = mask + (int64_t)row * t;
+  const int seg = (t + 63) / 64, i0 = min(lane * seg, t), i1 = min(i0 + seg, t);
+  int valid = 0;
+  float sum_em = 0.f, sum_m = 0.f;
+  for (int i = i0; i < i1; ++i) {
+    const float mk = m[i];
+    valid += mk == 1.f ? 1 : 0;
+    sum_em = fmaf(e[i], mk, sum_em);
+    sum_m += mk;
+  }
+  int before = valid;                                   // inclusive prefix over lanes ...
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int v = __shfl_up(before, o);
+    if (lane >= o) before += v;
+  }
+  int cum = before - valid;                             // ... valid tokens before this lane's piece
+  float win_e = 0.f, win_n = 0.f;
+  for (int i = i0; i < i1; ++i) {
+    if (m[i] == 1.f) {
+      ++cum;
+      if (cum >= 4 && cum <= 100) { win_e += e[i]; win_n += 1.f; }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    sum_em += __shfl_xor(sum_em, o);
+    sum_m += __shfl_xor(sum_m, o);
+    win_e += __shfl_xor(win_e, o);
+    win_n += __shfl_xor(win_n, o);
+  }
+  if (lane == 0) {
+    entropy[row] = sum_em / sum_m;
+    entropy_loss[row] = win_e / win_n;
   }
 }
 

@@ -176,14 +176,13 @@ class _Prepared:
             out["token_count"] = self.mask.sum().to(torch.int32)
             return out
         if self.seq_shape is not None:
+            # per-sample masked mean entropy (:141-143) and its tokens-4..100 window (:148-157): one kernel
             b, t = self.seq_shape
-            ent = self.ent.reshape(b, t)
-            m = self.mask.reshape(b, t)
-            out["entropy"] = (ent * m).sum(-1) / m.sum(-1)                    # :141-143
-            valid = m == 1
-            cum = torch.cumsum(valid, dim=-1)
-            win = (valid & (cum >= 4) & (cum <= 100)).to(torch.float32)      # :148-153
-            out["entropy_loss"] = (ent * win).sum(-1) / win.sum(-1)          # :155-157
+            stats = torch.empty((2, b), dtype=torch.float32, device=self.device)
+            with torch.cuda.device(self.device):
+                _lib.check(_lib.load().mj_grpo_sequence_entropy(
+                    _ptr(self.ent), _ptr(self.mask), b, t, stats[0].data_ptr(), stats[1].data_ptr(), self.stream()))
+            out["entropy"], out["entropy_loss"] = stats[0], stats[1]
         if return_token_entropy:
             out["token_entropy"] = self.ent.reshape(shape)
         if self.desc.inv_entropy_count != 0.0:

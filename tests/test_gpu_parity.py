@@ -330,3 +330,30 @@ def test_temperature_divides_logp_and_tempers_the_entropy(temp):
     plain = O.grpo_loss(hid.float().numpy(), w.float().numpy(), y.numpy(), None, np.zeros(520), np.ones(520), with_grads=False)
     np.testing.assert_allclose(met["per_token_logps"].reshape(-1), plain["per_token_logps"] / temp, atol=1e-3)
     assert np.abs(met["token_entropy"].reshape(-1) - plain["token_entropy"]).max() > 0.05      # it is a different entropy
+
+
+@pytest.mark.parametrize("b,t", [(3, 4), (5, 37), (4, 64), (7, 130), (2, 1000), (1, 7001)])
+def test_sequence_entropy_kernel_against_oracle(b, t):
+    """mj_grpo_sequence_entropy (train_modules/__init__.py:141-157) on masks that are not prefixes:
+    interleaved zeros, rows with fewer than four valid tokens (window empty: nan), an empty row."""
+    from mllm_jax_amd import _lib
+    d = _dev()
+    g = torch.Generator().manual_seed(100 * b + t)
+    ent = torch.rand(b, t, generator=g) * 5
+    mask = (torch.rand(b, t, generator=g) < 0.6).float()
+    mask[0, :] = 0
+    mask[0, : min(3, t)] = 1                      # three valid tokens: the 4..100 window is empty
+    if b > 1:
+        mask[1, :] = 0                            # empty row
+    ref_e, ref_w = O.sequence_entropy_stats(ent.double().numpy().reshape(-1), mask.numpy().reshape(-1), (b, t))
+    ent_d, mask_d = ent.to(d), mask.to(d)
+    out = torch.empty(2, b, device=d)
+    _lib.check(_lib.load().mj_grpo_sequence_entropy(ent_d.data_ptr(), mask_d.data_ptr(), b, t, out[0].data_ptr(),
+                                                    out[1].data_ptr(), torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    got_e, got_w = out[0].cpu().numpy(), out[1].cpu().numpy()
+    np.testing.assert_array_equal(np.isnan(got_e), np.isnan(ref_e))
+    np.testing.assert_array_equal(np.isnan(got_w), np.isnan(ref_w))
+    np.testing.assert_allclose(got_e[~np.isnan(ref_e)], ref_e[~np.isnan(ref_e)], rtol=1e-5)
+    np.testing.assert_allclose(got_w[~np.isnan(ref_w)], ref_w[~np.isnan(ref_w)], rtol=1e-5)
+    assert np.isnan(got_w[0])
