@@ -15,6 +15,7 @@ from __future__ import annotations
 import contextlib
 import ctypes as C
 import threading
+import weakref
 from typing import Any, Callable, Mapping, Optional
 
 import torch
@@ -40,6 +41,30 @@ def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
 def release_workspaces() -> None:
     """Drops the cached workspaces (one per device and stream)."""
     _workspaces.clear()
+
+
+_bf16_copies: dict = {}      # id(tensor) -> (weak reference to it, state key, bf16 copy)
+
+
+def _bf16_weights(w: torch.Tensor) -> torch.Tensor:
+    """bf16 view of the lm_head for the kernels.  The reference keeps float32 master weights and
+    casts per call (param_dtype f32, dtype bf16: MLLM_JAX/language/llama/llama.py:251-256); a cast of
+    [H,V] is a 3.3 GB pass at the Qwen2.5-7B shape, so the copy is kept for as long as the same
+    tensor object has not been written to (micro-batches and PPO epochs between two optimizer
+    steps) and dropped when that tensor dies."""
+    if w.dtype == torch.bfloat16:
+        return w.detach()
+    ident = id(w)                        # the caller's tensor object (detach() makes a new one per call)
+    key = (w._version, w.data_ptr(), tuple(w.shape), tuple(w.stride()))
+    hit = _bf16_copies.get(ident)
+    if hit is not None and hit[0]() is w and hit[1] == key:
+        return hit[2]
+    copy = w.detach().to(torch.bfloat16)
+    try:
+        _bf16_copies[ident] = (weakref.ref(w, lambda _r, i=ident: _bf16_copies.pop(i, None)), key, copy)
+    except TypeError:                    # objects that cannot be weakly referenced: no cache
+        pass
+    return copy
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -77,7 +102,7 @@ class _Prepared:
         dev = hidden.device
         self.n, self.h, self.v, self.seq_shape, self.device = n, h, v, seq_shape, dev
         self.hidden = self._operand(hidden.to(torch.bfloat16))
-        self.w = self._operand(lm_head.detach().to(torch.bfloat16))
+        self.w = self._operand(_bf16_weights(lm_head))
         self.targets = torch.as_tensor(target_ids, device=dev).reshape(-1).to(torch.int32).contiguous()
         if self.targets.numel() != n:
             raise ValueError(f"target_ids has {self.targets.numel()} elements, expected {n}")

@@ -357,3 +357,59 @@ def test_sequence_entropy_kernel_against_oracle(b, t):
     np.testing.assert_allclose(got_e[~np.isnan(ref_e)], ref_e[~np.isnan(ref_e)], rtol=1e-5)
     np.testing.assert_allclose(got_w[~np.isnan(ref_w)], ref_w[~np.isnan(ref_w)], rtol=1e-5)
     assert np.isnan(got_w[0])
+
+
+def _shifted_case(seed, shift):
+    n, h, v, b = 768, 64, 1000, 3
+    hid, w, y, adv, mask = _case(seed, n, h, v, b)
+    w = w.float(); w[0, :] = 1.0
+    hid = hid.float(); hid[:, 0] = 0.0; hid[256:512, 0] = shift      # second 256-token chunk out of the exp window
+    return hid.to(torch.bfloat16), w.to(torch.bfloat16), y, adv, mask, (n, h, v, b)
+
+
+def test_rescue_pass_with_token_compaction_and_sft():
+    """The on-device rescue (running-maximum pass for a chunk whose logsumexp leaves the exp window)
+    together with the options that change what the chunk kernels see: compacted tokens, the SFT flag."""
+    import mllm_jax_amd as M
+    d = _dev()
+    hid, w, y, adv, mask, (n, h, v, b) = _shifted_case(23, 90.0)
+    old = _old_from(_ref_logp(hid, w, y), 24)
+    ref = O.grpo_loss(hid.float().numpy(), w.float().numpy(), y.numpy(), old.numpy(), adv.numpy(), mask.numpy())
+    met, (dh, dw) = M.grpo_loss_value_and_grad(hid.to(d), w.to(d), y.to(d), old.to(d), adv.to(d), mask.to(d),
+                                               chunk_tokens=256, skip_masked=True)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(met["per_token_logps"].cpu().numpy().reshape(-1), ref["per_token_logps"], atol=LOGP_ATOL, rtol=0)
+    assert abs(met["loss"].item() - ref["loss"]) <= LOSS_RTOL * abs(ref["loss"])
+    assert _rel(dh.float().cpu().numpy(), ref["d_hidden"]) <= GRAD_RTOL
+    assert _rel(dw.cpu().numpy(), ref["d_lm_head"]) <= GRAD_RTOL
+    sref = O.sft_cross_entropy(hid.float().numpy(), w.float().numpy(), y.numpy(), mask.numpy())
+    hp, wp = hid.to(d).requires_grad_(), w.to(d).requires_grad_()
+    out = M.sft_fused_loss(hp, wp, y.to(d), mask.to(d), chunk_tokens=256)
+    out["loss"].backward()
+    torch.cuda.synchronize()
+    assert abs(out["loss"].item() - sref["loss"]) <= LOSS_RTOL * abs(sref["loss"])
+    assert _rel(hp.grad.float().cpu().numpy(), sref["d_hidden"]) <= GRAD_RTOL
+    assert _rel(wp.grad.float().cpu().numpy(), sref["d_lm_head"]) <= GRAD_RTOL
+
+
+def test_rescue_pass_in_the_workspace_free_forward():
+    import ctypes as C
+    from mllm_jax_amd import _lib
+    d = _dev()
+    hid, w, y, adv, mask, (n, h, v, b) = _shifted_case(25, -95.0)
+    ref = O.grpo_loss(hid.float().numpy(), w.float().numpy(), y.numpy(), None, adv.numpy(), mask.numpy(), with_grads=False)
+    desc = _lib.MjGrpoDesc()
+    desc.n_tokens, desc.hidden, desc.vocab, desc.ld_hidden, desc.ld_w, desc.chunk_tokens = n, h, v, h, v, 256
+    desc.eps_low, desc.eps_high, desc.temperature = 0.2, 0.3, 1.0
+    desc.inv_total_valid_tokens, desc.grad_loss_scale = 1.0 / float(mask.sum()), 1.0
+    t = lambda x, dt: x.to(d).to(dt).contiguous()
+    hid_d, w_d, y_d, adv_d, mask_d = t(hid, torch.bfloat16), t(w, torch.bfloat16), t(y, torch.int32), t(adv, torch.float32), t(mask, torch.float32)
+    logp, lse, ent = (torch.empty(n, device=d) for _ in range(3))
+    loss = torch.empty(2, device=d)
+    _lib.check(_lib.load().mj_grpo_forward_noalloc(C.byref(desc), hid_d.data_ptr(), w_d.data_ptr(), y_d.data_ptr(), None,
+                                                   adv_d.data_ptr(), mask_d.data_ptr(), logp.data_ptr(), lse.data_ptr(),
+                                                   ent.data_ptr(), loss.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(logp.cpu().numpy(), ref["per_token_logps"], atol=LOGP_ATOL, rtol=0)
+    np.testing.assert_allclose(lse.cpu().numpy(), ref["lse"], atol=2e-3, rtol=0)
+    assert abs(loss[0].item() - ref["loss"]) <= LOSS_RTOL * abs(ref["loss"]) + 1e-7

@@ -203,3 +203,35 @@ def test_separate_backward_refuses_entropy_bonus():
     st = lib.mj_grpo_backward(C.byref(d), p, p, p, p, p, p, p, p, p, p, ws.data_ptr(), both, None)
     assert st == 5      # MJ_GRPO_ERR_UNSUPPORTED
     assert b"entropy" in lib.mj_grpo_last_error()
+
+
+def test_value_head_with_the_rescue_pass():
+    """entropy_coef = 0 (E-based backward) with logits far outside the exp window: the running-maximum
+    pass takes over on the device; dv * value_w still joins d_hidden."""
+    import mllm_jax_amd as M
+    dev = torch.device("cuda:0")
+    b, l, h, v = 4, 65, 64, 520
+    ids, emb, pos, w, wv, bv, labels, adv = _batch(14, b, l, h, v)
+    t = l - 1
+    hidden = (emb[ids].float() + pos[None].float())
+    w = w.float(); w[0, :] = 1.0
+    hidden[..., 0] = 80.0                                    # every logit shifted by +80
+    hidden, w = hidden.to(torch.bfloat16), w.to(torch.bfloat16)
+    g = torch.Generator().manual_seed(15)
+    hid_flat = hidden[:, :-1].reshape(b * t, h).float().numpy()
+    vp_ref = hid_flat.astype(np.float64) @ wv.double().numpy() + float(bv)
+    r = torch.from_numpy(vp_ref).float() + torch.randn(b * t, generator=g)
+    hd, wd = hidden.to(dev).requires_grad_(), w.to(dev).requires_grad_()
+    wvd, bvd = wv.to(dev).requires_grad_(), bv.to(dev).requires_grad_()
+    module = M.PPOActorCriticModule(lambda input_ids, attention_mask: hd, wd, (wvd, bvd))
+    out = module({"input_ids": ids.to(dev), "attention_mask": torch.ones(b, l, device=dev), "labels": labels.to(dev),
+                  "advantages": adv.to(dev), "returns": r.reshape(b, t).to(dev)})
+    out["loss"].backward()
+    torch.cuda.synchronize()
+    ref = O.ppo_actor_critic_loss(hid_flat, w.float().numpy(), wv.numpy(), float(bv), ids[:, 1:].reshape(-1).numpy(), None,
+                                  adv.reshape(-1).numpy(), labels[:, 1:].reshape(-1).float().numpy(), returns=r.numpy())
+    assert abs(ref["lse"].mean() - 80) < 15 if "lse" in ref else True
+    assert abs(float(out["loss"].detach()) - ref["loss"]) <= LOSS_RTOL * abs(ref["loss"]) + 2e-6
+    assert _rel(hd.grad[:, :-1].reshape(b * t, h).float().cpu().numpy(), ref["d_hidden"]) <= GRAD_RTOL
+    assert _rel(wd.grad.float().cpu().numpy(), ref["d_lm_head"]) <= GRAD_RTOL
+    assert _rel(wvd.grad.cpu().numpy(), ref["d_value_w"]) <= GRAD_RTOL

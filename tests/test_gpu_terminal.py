@@ -78,3 +78,23 @@ def test_accumulating_with_a_scaled_loss_poisons_the_accumulator():
         out["loss"].backward()
     torch.cuda.synchronize()
     assert _rel(acc.cpu().numpy(), ref["d_lm_head"]) <= GRAD_RTOL
+
+
+def test_bf16_copy_of_float32_weights_is_reused_until_they_change():
+    import mllm_jax_amd as M
+    from mllm_jax_amd import loss as L
+    ref, hp, wp, args = _setup(54)
+    a = L._bf16_weights(wp)
+    assert a.dtype == torch.bfloat16 and L._bf16_weights(wp) is a            # same tensor, same version: reused
+    out1 = M.grpo_fused_loss(hp, wp, *args)["loss"].item()
+    with torch.no_grad():
+        wp.mul_(1.5)                                                          # an optimizer step writes in place
+    b = L._bf16_weights(wp)
+    assert b is not a and torch.equal(b, wp.detach().to(torch.bfloat16))
+    out2 = M.grpo_fused_loss(hp, wp, *args)["loss"].item()
+    assert out1 == out2 == pytest.approx(ref["loss"], rel=1e-3)               # on-policy: the loss does not depend on W
+    lp1 = M.grpo_fused_loss(hp, wp, *args)["per_token_logps"]
+    with torch.no_grad():
+        wp.mul_(0.5)
+    lp2 = M.grpo_fused_loss(hp, wp, *args)["per_token_logps"]
+    assert not torch.equal(lp1, lp2)                                          # the stale copy is not used
