@@ -293,7 +293,9 @@ def main() -> int:
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                 "avg_launch_ms": round(avg_launch_ms, 3), "launches": dom_launches,
                 "flop_per_launch": flop_per_launch,
-                "traffic": None if args.chunk_tokens else MEASURED_TRAFFIC_BYTES.get((args.config, dom))}
+                "traffic": None if args.chunk_tokens else MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
+                "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this bench, summary in "
+                                  "profiles/cfg2_qwen7b_fused_fwd_bwd.txt (not re-measured in this run)"}
 
     line = {
         "metric": "grpo_fused_loss_fwd_bwd_tokens_per_s", "value": round(tokens_per_s, 1), "unit": "tokens/s",

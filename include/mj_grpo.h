@@ -110,7 +110,9 @@ int mj_grpo_forward(const MjGrpoDesc* desc, const void* hidden, const void* lm_h
  * does not fit even with 256-token chunks (12 bytes per token plus 6 * ceil(V/256) * 4 bytes per
  * token of a chunk) are refused with MJ_GRPO_ERR_WORKSPACE.  All calls on one device share the
  * array: calls that overlap on a device (two streams, two threads) race; serialise them.  Outputs
- * are those of mj_grpo_forward bit for bit. */
+ * are those of mj_grpo_forward bit for bit.  The first call on a device looks the array's address
+ * up (hipGetSymbolAddress) and raises the kernels' LDS limit (hipFuncSetAttribute): make one call
+ * outside stream capture before capturing others. */
 #define MJ_GRPO_NOALLOC_SCRATCH_BYTES (32u << 20)
 int mj_grpo_forward_noalloc(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
                             const int32_t* targets, const float* old_logp, const float* advantages,
