@@ -1,5 +1,6 @@
 """GPU: the fused call is capturable in a HIP graph (no allocation, no memset, no host
-synchronisation inside the library) and every replay reproduces the eager result bit for bit."""
+synchronisation inside the library) and every replay reproduces the eager result bit for bit,
+including replays whose data send one chunk through the on-device rescue pass."""
 import pytest
 import torch
 
@@ -33,8 +34,14 @@ def test_graph_replays_match_eager(skip_masked):
         with torch.cuda.graph(graph, stream=side):
             met, (dh, dw) = call(static)
     torch.cuda.synchronize()
-    for rep in range(3):
+    for rep in range(4):
         new = fresh()
+        if rep in (1, 2):
+            # every logit of the second 256-token chunk shifted by +90: that chunk's range check fails
+            # on the device and the captured running-maximum launches do the work in this replay only
+            new[1][0, :] = 1.0
+            new[0][:, 0] = 0.0
+            new[0][256:512, 0] = 90.0 if rep == 1 else -90.0
         for s, t in zip(static, new):
             s.copy_(t)
         torch.cuda.synchronize()
