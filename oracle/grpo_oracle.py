@@ -36,6 +36,9 @@ Parity unpinned (documented, accepted):
   * JAX's half-gradient tie rule exactly at ratio == 1-eps_low / 1+eps_high
     (lax.min / lax.clip JVP); the closed form here takes the full unclipped
     gradient on the closed interval.
+  * Target ids outside [0, V): jnp.take_along_axis wraps negative ids and yields NaN
+    past V; the oracle is only ever called with ids in range (the kernels clamp such
+    ids, and their tests compare against the oracle on the clamped ids).
 """
 from __future__ import annotations
 
