@@ -184,6 +184,8 @@ def main() -> int:
     ap.add_argument("--entropy-coef", type=float, default=0.0,
                     help="add PPO's entropy bonus (plugins/training/ppo/module.py:140): times the running-maximum "
                          "kernels + the in-place dZ pass instead of the default path")
+    ap.add_argument("--dw-dtype", choices=("f32", "bf16"), default="f32",
+                    help="dtype of the lm_head gradient the dW kernel writes (the reference's is float32: the default)")
     ap.add_argument("--no-kernel-events", action="store_true",
                     help="time the steps without the per-kernel HIP events (each event pair leaves ~10 us between "
                          "two kernels: nothing at the headline shape, 10 %% of a step at the smallest); the per-kernel "
@@ -222,6 +224,8 @@ def main() -> int:
     kw = dict(epsilon_low=cfg.eps_low, epsilon_high=cfg.eps_high, final_logit_softcap=cfg.softcap,
               chunk_tokens=args.chunk_tokens or None, dhidden_splits=args.dhidden_splits)
     step_kw = dict(entropy_coef=args.entropy_coef) if args.entropy_coef else {}
+    if args.dw_dtype == "bf16":
+        step_kw["lm_head_grad_dtype"] = torch.bfloat16
 
     def logp_fn(wl):
         with torch.no_grad():
@@ -305,7 +309,7 @@ def main() -> int:
         "config": {"workload": f"BASELINE configs[{args.config}] {cfg.name}: fused GRPO loss fwd+bwd, "
                                f"{n} tokens x hidden {h} x vocab {v}", "tokens": n, "hidden": h, "vocab": v,
                    "chunk_tokens": args.chunk_tokens or min(16384, n), "softcap": cfg.softcap,
-                   "ld_w": v + args.pad_w, "dhidden_splits": args.dhidden_splits or "auto",
+                   "ld_w": v + args.pad_w, "dhidden_splits": args.dhidden_splits or "auto", "dw_dtype": args.dw_dtype,
                    "eps": [cfg.eps_low, cfg.eps_high]},
         "pct_bf16_mfma_peak": round(100.0 * mfu, 2),
         "algorithmic_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 1),

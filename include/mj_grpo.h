@@ -48,13 +48,20 @@ enum {
   MJ_GRPO_FLAG_SFT = 1u << 1,           /* masked cross-entropy instead of the clipped surrogate
                                            (plugins/sft/jax/sft_module.py:22-45): per-token loss
                                            -logp, advantages/old_logp ignored */
-  MJ_GRPO_FLAG_SKIP_MASKED = 1u << 2    /* tokens whose gradient is zero by construction (mask 0: prompt
+  MJ_GRPO_FLAG_SKIP_MASKED = 1u << 2,   /* tokens whose gradient is zero by construction (mask 0: prompt
                                            and padding positions, labels of train_modules/__init__.py:120;
                                            advantage 0 when nothing else feeds the gradient) are moved
                                            behind the others and left out of the backward products.
                                            Same outputs (d_lm_head up to summation order); the forward
                                            still covers every token.  No counterpart in the reference,
                                            which multiplies the zeros.  Needs a larger workspace. */
+  MJ_GRPO_FLAG_DW_BF16 = 1u << 3        /* d_lm_head is a bf16 [H, ld_w] matrix instead of a float one (for
+                                           callers whose lm_head parameter, and so its gradient, is bf16;
+                                           the reference's parameter gradients are float32,
+                                           llama/llama.py:251-256).  Each entry is summed in fp32 and rounded
+                                           once per call and per chunk of chunk_tokens; with
+                                           MJ_GRPO_FLAG_DW_ACCUMULATE the value in memory is added in fp32
+                                           before that rounding. */
 };
 
 typedef struct MjGrpoDesc {
@@ -122,7 +129,7 @@ int mj_grpo_forward_noalloc(const MjGrpoDesc* desc, const void* hidden, const vo
 /* Forward and backward in one pass (executes 6*N*H*V flop).  Replaces
  * jax.value_and_grad(loss_fn) of plugins/training/update/train_step.py:15-24 restricted to
  * the lm_head + loss part: besides the forward outputs it writes
- * d_hidden[N, ld_hidden] bf16 and d_lm_head[H, ld_w] f32, both already multiplied by
+ * d_hidden[N, ld_hidden] bf16 and d_lm_head[H, ld_w] f32 (bf16 with MJ_GRPO_FLAG_DW_BF16), both already multiplied by
  * grad_loss_scale.  The workspace holds 16-bit (half) logits for chunk_tokens tokens at a time.
  * With entropy_coef != 0 the gradient includes the entropy bonus,
  * d(-coef*entropy)/dz = coef * mask * inv_entropy_count * p * (log p + H_t). */
@@ -130,7 +137,7 @@ int mj_grpo_forward_backward(const MjGrpoDesc* desc, const void* hidden, const v
                              const int32_t* targets, const float* old_logp,
                              const float* advantages, const float* mask, float* logp,
                              float* lse, float* token_entropy, float* loss, void* d_hidden,
-                             float* d_lm_head, void* workspace, size_t workspace_bytes,
+                             void* d_lm_head, void* workspace, size_t workspace_bytes,
                              void* stream);
 
 /* The two per-sequence entropy entries of the reference's return dict
@@ -172,7 +179,7 @@ int mj_grpo_value_workspace_bytes(const MjGrpoDesc* desc, size_t* extra_bytes);
 int mj_grpo_forward_backward_value(const MjGrpoDesc* desc, const MjPpoValue* value, const void* hidden,
                                    const void* lm_head, const int32_t* targets, const float* old_logp,
                                    const float* advantages, const float* mask, float* logp, float* lse,
-                                   float* token_entropy, float* loss, void* d_hidden, float* d_lm_head,
+                                   float* token_entropy, float* loss, void* d_hidden, void* d_lm_head,
                                    void* workspace, size_t workspace_bytes, void* stream);
 
 /* The value head alone (PPOActorCriticModule.value, module.py:55-57): values[n] = hidden . value_w + value_b. */
@@ -186,7 +193,7 @@ int mj_value_head_forward(const void* hidden, int64_t ld_hidden, const float* va
 int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
                      const int32_t* targets, const float* old_logp, const float* advantages,
                      const float* mask, const float* lse, const float* logp, void* d_hidden,
-                     float* d_lm_head, void* workspace, size_t workspace_bytes, void* stream);
+                     void* d_lm_head, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Sequence-level advantage estimators on the device (host NumPy in the reference, evaluated by the
  * runner at runner/grpo_gsm8k.py:680).  rewards, advantages: float32 [b]; group_ids: int32 [b] (any

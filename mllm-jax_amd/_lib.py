@@ -14,6 +14,7 @@ OK = 0
 FLAG_DW_ACCUMULATE = 1 << 0
 FLAG_SFT = 1 << 1
 FLAG_SKIP_MASKED = 1 << 2
+FLAG_DW_BF16 = 1 << 3
 
 EXPORTS = ("mj_grpo_version", "mj_grpo_last_error", "mj_grpo_workspace_bytes", "mj_grpo_forward",
            "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_forward_noalloc", "mj_grpo_probe_mfma", "mj_grpo_forward_backward_value",

@@ -105,7 +105,7 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
     return fail(MJ_GRPO_ERR_UNSUPPORTED, "an entropy bonus needs temperature 1 (got %g)", (double)d->temperature);
   if (d->softcap < 0.f || !isfinite(d->softcap)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "softcap must be >= 0");
   if (d->chunk_tokens < 0) return fail(MJ_GRPO_ERR_SHAPE, "chunk_tokens must be >= 0");
-  if (d->flags & ~(uint32_t)(MJ_GRPO_FLAG_DW_ACCUMULATE | MJ_GRPO_FLAG_SFT | MJ_GRPO_FLAG_SKIP_MASKED))
+  if (d->flags & ~(uint32_t)(MJ_GRPO_FLAG_DW_ACCUMULATE | MJ_GRPO_FLAG_SFT | MJ_GRPO_FLAG_SKIP_MASKED | MJ_GRPO_FLAG_DW_BF16))
     return fail(MJ_GRPO_ERR_UNSUPPORTED, "unknown bits in flags (0x%x)", d->flags);
   if (!isfinite(d->inv_total_valid_tokens)) return fail(MJ_GRPO_ERR_SHAPE, "inv_total_valid_tokens not finite");
   if (!isfinite(d->entropy_coef) || !isfinite(d->inv_entropy_count) || d->inv_entropy_count < 0.f)
@@ -188,12 +188,13 @@ enum Mode { kForward, kForwardBackward, kBackwardOnly };
 int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head, const int32_t* targets,
         const float* old_logp, const float* adv, const float* mask, float* logp, float* lse,
         float* ent, float* loss, const float* saved_lse, const float* saved_logp, void* d_hidden,
-        float* d_w, void* workspace, size_t ws_bytes, void* stream_v, const MjPpoValue* pv = nullptr) {
+        void* d_w, void* workspace, size_t ws_bytes, void* stream_v, const MjPpoValue* pv = nullptr) {
   Plan p;
   int rc = make_plan(d, &p);
   if (rc) return rc;
   const bool sft = (d->flags & MJ_GRPO_FLAG_SFT) != 0;
   const bool bwd = mode != kForward;
+  const bool dw_bf16 = (d->flags & MJ_GRPO_FLAG_DW_BF16) != 0;
   if (!hidden || !lm_head || !targets || !mask) return fail(MJ_GRPO_ERR_NULL, "hidden/lm_head/targets/mask is NULL");
   if (!sft && !adv) return fail(MJ_GRPO_ERR_NULL, "advantages is NULL");
   if (mode != kBackwardOnly && (!logp || !lse || !loss)) return fail(MJ_GRPO_ERR_NULL, "logp/lse/loss output is NULL");
@@ -254,7 +255,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
   }
   if (bwd) {
     if ((rc = enable_lds(mj::k_dhidden<BM, BN>))) return rc;
-    if ((rc = enable_lds(mj::k_dw<BM, BN>))) return rc;
+    if ((rc = dw_bf16 ? enable_lds(mj::k_dw<BM, BN, true>) : enable_lds(mj::k_dw<BM, BN, false>))) return rc;
   }
 
   // Value head (PPO critic), on the caller's token order: value_pred, the clipped value loss and
@@ -430,7 +431,8 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       const mj::TileMap mw = mj::TileMap::pick_shape((V + BM - 1) / BM, (H + BN - 1) / BN, 0, 1);
       {
         Timed t(MJ_GRPO_K_DW, st);
-        mj::k_dw<BM, BN><<<mw.items(), mj::kThreads, lds, st>>>(w, mw);
+        if (dw_bf16) mj::k_dw<BM, BN, true><<<mw.items(), mj::kThreads, lds, st>>>(w, mw);
+        else mj::k_dw<BM, BN, false><<<mw.items(), mj::kThreads, lds, st>>>(w, mw);
       }
     }
     if ((rc = check_launch("chunk kernels"))) return rc;
@@ -527,7 +529,7 @@ int mj_grpo_forward(const MjGrpoDesc* desc, const void* hidden, const void* lm_h
 int mj_grpo_forward_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
                              const int32_t* targets, const float* old_logp, const float* advantages,
                              const float* mask, float* logp, float* lse, float* token_entropy, float* loss,
-                             void* d_hidden, float* d_lm_head, void* workspace, size_t workspace_bytes,
+                             void* d_hidden, void* d_lm_head, void* workspace, size_t workspace_bytes,
                              void* stream) {
   return run(kForwardBackward, desc, hidden, lm_head, targets, old_logp, advantages, mask, logp, lse,
              token_entropy, loss, nullptr, nullptr, d_hidden, d_lm_head, workspace, workspace_bytes, stream);
@@ -552,7 +554,7 @@ int mj_grpo_value_workspace_bytes(const MjGrpoDesc* desc, size_t* extra_bytes) {
 int mj_grpo_forward_backward_value(const MjGrpoDesc* desc, const MjPpoValue* value, const void* hidden,
                                    const void* lm_head, const int32_t* targets, const float* old_logp,
                                    const float* advantages, const float* mask, float* logp, float* lse,
-                                   float* token_entropy, float* loss, void* d_hidden, float* d_lm_head,
+                                   float* token_entropy, float* loss, void* d_hidden, void* d_lm_head,
                                    void* workspace, size_t workspace_bytes, void* stream) {
   if (value == nullptr) return fail(MJ_GRPO_ERR_NULL, "value is NULL (use mj_grpo_forward_backward)");
   return run(kForwardBackward, desc, hidden, lm_head, targets, old_logp, advantages, mask, logp, lse, token_entropy,
@@ -573,7 +575,7 @@ int mj_value_head_forward(const void* hidden, int64_t ld_hidden, const float* va
 
 int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_head, const int32_t* targets,
                      const float* old_logp, const float* advantages, const float* mask, const float* lse,
-                     const float* logp, void* d_hidden, float* d_lm_head, void* workspace,
+                     const float* logp, void* d_hidden, void* d_lm_head, void* workspace,
                      size_t workspace_bytes, void* stream) {
   return run(kBackwardOnly, desc, hidden, lm_head, targets, old_logp, advantages, mask, nullptr, nullptr,
              nullptr, nullptr, lse, logp, d_hidden, d_lm_head, workspace, workspace_bytes, stream);
@@ -831,5 +833,6 @@ template __global__ void mj::k_logits_stats<256, 256, mj::kStatsMax, false>(mj::
 template __global__ void mj::k_logits_stats<256, 256, mj::kStatsMax, true>(mj::LogitsArgs, mj::TileMap);
 template __global__ void mj::k_logits_stats<256, 256, mj::kStatsGrad, false>(mj::LogitsArgs, mj::TileMap);
 template __global__ void mj::k_dhidden<256, 256>(mj::DhArgs, mj::TileMap);
-template __global__ void mj::k_dw<256, 256>(mj::DwArgs, mj::TileMap);
+template __global__ void mj::k_dw<256, 256, false>(mj::DwArgs, mj::TileMap);
+template __global__ void mj::k_dw<256, 256, true>(mj::DwArgs, mj::TileMap);
 template __global__ void mj::k_logits_rows<256, 256>(mj::LogitsRowsArgs, mj::TileMap);

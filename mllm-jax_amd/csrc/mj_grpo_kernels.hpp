@@ -726,7 +726,7 @@ struct DwArgs {
   const __bf16* hs;    // [n, H]: rs * hidden, the token-side operand while state == 0
   int64_t ld_z, ld_hid;
   int H, V, n;         // n = tokens of the chunk
-  float* dw;           // [H, ld_dw] f32
+  void* dw;            // [H, ld_dw]: f32, or bf16 in the BF16OUT kernel
   int64_t ld_dw;
   int accumulate;
   const int* n_live;   // see live_pad
@@ -737,7 +737,9 @@ struct DwArgs {
 // Tile of dW^T: rows = vocab (MFMA row direction), columns = hidden (lanes).  A lane's four
 // consecutive accumulator rows are four consecutive floats of one dW row: 16-byte accesses.
 // Both operands are token-major in memory, so both go through the transposing LDS read.
-template <int BM, int BN>
+// BF16OUT: dW is a bf16 matrix; two lanes exchange halves (store_rows8) so that each writes eight
+// consecutive entries of one row, and an accumulating call adds in fp32 and rounds once.
+template <int BM, int BN, bool BF16OUT>
 __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
   using G = GemmTN<BM, BN, kKRow, kKRow, 2>;   // two slices in flight: measured 2-3% faster here, not in the other products
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -757,9 +759,53 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
   // address is (its hidden row) * ld + (its 4-float group), the vocab block is the scalar offset.
   const int h0 = n0 + wn * G::WN, v0 = m0 + wm * G::WM;
   const int hrows = min(max(p.H - h0, 0), G::WN);
+  const int vleft = p.V - v0;                            // V % 8 == 0: groups of 4 or 8 are in or out together
+  if (BF16OUT) {
+    const uint32_t ld2 = (uint32_t)p.ld_dw * 2;
+    const __amdgpu_buffer_rsrc_t rs =
+        make_rsrc_wave((uint16_t*)p.dw + (int64_t)h0 * p.ld_dw + v0, (int64_t)hrows * ld2 - (int64_t)v0 * 2);
+#pragma unroll
+    for (int ni = 0; ni < G::NI; ++ni) {
+      const uint32_t lane_off = (uint32_t)((ni * 32 + l31) * ld2 + lhi * 16);   // the lane's 16 of a pair's 32 bytes
+      u32x4 old[G::MI][2];
+      if (p.accumulate) {                     // all loads of this column block before its first store
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int qp = 0; qp < 2; ++qp) {
+            const int vv = mi * 32 + qp * 16;
+            old[mi][qp] = __builtin_amdgcn_raw_buffer_load_b128(rs, (vv + lhi * 8) < vleft ? lane_off : kOob,
+                                                                (uint32_t)vv * 2, 0);
+          }
+      }
+#pragma unroll
+      for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+        for (int qp = 0; qp < 2; ++qp) {
+          const int vv = mi * 32 + qp * 16;
+          float v[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) v[j] = g.acc[mi][ni][qp * 8 + j];
+          if (p.accumulate) {
+            // undo the exchange of store_rows8 on what is in memory (the exchange is its own inverse)
+            const u32x4 o = old[mi][qp];
+            const auto s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
+            const uint32_t w[4] = {s0[0], s1[0], s0[1], s1[1]};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              v[2 * j] += __uint_as_float(w[j] << 16);
+              v[2 * j + 1] += __uint_as_float(w[j] & 0xffff0000u);
+            }
+          }
+          store_rows8<false>(v, 0xffffffffu, rs, (vv + lhi * 8) < vleft ? lane_off : kOob, (uint32_t)vv * 2);
+        }
+    }
+    return;
+  }
   const uint32_t ld4 = (uint32_t)p.ld_dw * 4;
-  const __amdgpu_buffer_rsrc_t rs = make_rsrc_wave(p.dw + (int64_t)h0 * p.ld_dw + v0, (int64_t)hrows * ld4 - (int64_t)v0 * 4);
-  const int vleft = p.V - v0;                            // V % 8 == 0: groups of 4 are in or out together
+  const __amdgpu_buffer_rsrc_t rs =
+      make_rsrc_wave((float*)p.dw + (int64_t)h0 * p.ld_dw + v0, (int64_t)hrows * ld4 - (int64_t)v0 * 4);
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
     const uint32_t lane_off = (uint32_t)((ni * 32 + l31) * ld4 + lhi * 16);

@@ -168,7 +168,10 @@ class _Prepared:
                 _ptr(self.adv), _ptr(self.mask), _ptr(self.logp), _ptr(self.lse), _ptr(self.ent),
                 _ptr(self.loss), _ptr(ws), ws.numel(), self.stream()))
 
-    def forward_backward(self, d_w: Optional[torch.Tensor] = None, value: Optional["_ValueHead"] = None):
+    def forward_backward(self, d_w: Optional[torch.Tensor] = None, value: Optional["_ValueHead"] = None,
+                         dw_dtype: torch.dtype = torch.float32):
+        """One fused pass.  The lm_head gradient goes into `d_w` (float32 or bf16, laid out like
+        lm_head; added to when the descriptor says accumulate) or into a new tensor of `dw_dtype`."""
         _, both = _lib.workspace_bytes(self.desc)
         if value is not None:
             both += _lib.value_workspace_bytes(self.desc)
@@ -177,7 +180,13 @@ class _Prepared:
         ld = self.hidden.stride(0)
         d_h = torch.empty((self.n, ld), dtype=torch.bfloat16, device=self.device)[:, : self.h]
         if d_w is None:
-            d_w = torch.empty((self.h, self.w.stride(0)), dtype=torch.float32, device=self.device)
+            d_w = torch.empty((self.h, self.w.stride(0)), dtype=dw_dtype, device=self.device)
+        if d_w.dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"the lm_head gradient is float32 or bfloat16 (got {d_w.dtype})")
+        if d_w.dtype == torch.bfloat16:
+            self.desc.flags |= _lib.FLAG_DW_BF16
+        else:
+            self.desc.flags &= ~_lib.FLAG_DW_BF16
         with torch.cuda.device(self.device):
             if value is None:
                 _lib.check(_lib.load().mj_grpo_forward_backward(
@@ -252,13 +261,15 @@ _DEFAULTS = dict(total_valid_token_count=None, epsilon_low=0.2, epsilon_high=0.3
 
 
 def grpo_loss_value_and_grad(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
-                             return_token_entropy=False, accumulate_into=None, **kw):
+                             return_token_entropy=False, accumulate_into=None,
+                             lm_head_grad_dtype=torch.float32, **kw):
     """value_and_grad form of the loss, the call shape of the reference's train step
     (plugins/training/update/train_step.py:24): returns (metrics, (d_hidden, d_lm_head)).
 
     d_hidden is bf16 [N,H]; d_lm_head is float32 [H,V] (the reference's parameter gradients
-    are float32).  `accumulate_into` (a float32 [H,V] tensor) makes the kernel add into an
-    existing gradient buffer instead of overwriting (grad accumulation, train_step.py:30-33).
+    are float32) unless `lm_head_grad_dtype=torch.bfloat16` asks the dW kernel for a bf16 matrix.
+    `accumulate_into` (a float32 or bf16 [H,V] tensor) makes the kernel add into an existing
+    gradient buffer instead of overwriting (grad accumulation, train_step.py:30-33).
     One fused pass: 6*N*H*V flop, 16-bit logits of at most `chunk_tokens` tokens in the workspace.
     `entropy_coef` != 0 subtracts entropy_coef * sum(H_t*mask)/(sum(mask)+1e-8) from the loss
     (the entropy bonus of plugins/training/ppo/module.py:75-77, :140), gradient included; that
@@ -270,14 +281,15 @@ def grpo_loss_value_and_grad(hidden, lm_head, target_ids, old_logps, advantages,
                   accumulate=accumulate_into is not None, **opts)
     if accumulate_into is not None:
         _check_accumulator(accumulate_into, p)
-    d_h, d_w = p.forward_backward(accumulate_into)
+    d_h, d_w = p.forward_backward(accumulate_into, dw_dtype=lm_head_grad_dtype)
     return p.metrics(return_token_entropy), (d_h.reshape(hidden.shape), d_w)
 
 
 def _check_accumulator(buf: torch.Tensor, p: "_Prepared") -> None:
-    if buf.dtype != torch.float32 or tuple(buf.shape) != (p.h, p.v) \
+    if buf.dtype not in (torch.float32, torch.bfloat16) or tuple(buf.shape) != (p.h, p.v) \
             or buf.stride(1) != 1 or buf.stride(0) != p.w.stride(0) or buf.device != p.device:
-        raise ValueError("the lm_head gradient accumulator must be a float32 [H,V] device tensor laid out like lm_head")
+        raise ValueError("the lm_head gradient accumulator must be a float32 or bfloat16 [H,V] device tensor "
+                         "laid out like lm_head")
 
 
 class _CallMode(threading.local):
@@ -292,7 +304,7 @@ _accumulate_target = _CallMode()
 @contextlib.contextmanager
 def accumulate_lm_head_grad_into(buffer: torch.Tensor):
     """Within this context every differentiable fused-loss call ADDS its lm_head gradient into
-    `buffer` (float32 [H,V]) inside the dW kernel and hands autograd no lm_head gradient: the
+    `buffer` (float32 or bf16 [H,V]) inside the dW kernel and hands autograd no lm_head gradient: the
     grad-accumulation `ga + g` of plugins/training/update/train_step.py:30-33 without a
     separate [H,V] gradient tensor or a pass over it.  The loss must be terminal (it is
     differentiated with upstream gradient 1, as training_step does; any other upstream gradient
@@ -338,6 +350,8 @@ class _FusedLossFn(torch.autograd.Function):
         ctx.direct = ctx.terminal = False
         ctx.d_w = ctx.buf = ctx.value = None
         if want_grad:
+            # a bf16 parameter takes a bf16 gradient: the dW kernel writes it, no conversion pass
+            dw_dtype = torch.bfloat16 if lm_head.dtype == torch.bfloat16 else torch.float32
             buf = _accumulate_target.buffer if lm_head.requires_grad else None
             if buf is not None:
                 _check_accumulator(buf, prepared)
@@ -347,11 +361,11 @@ class _FusedLossFn(torch.autograd.Function):
                 ctx.direct, ctx.buf = True, buf
                 ctx.save_for_backward(d_h)
             elif _accumulate_target.terminal:
-                d_h, d_w = prepared.forward_backward(None, value)
+                d_h, d_w = prepared.forward_backward(None, value, dw_dtype)
                 ctx.terminal, ctx.d_w = True, d_w      # kept out of save_for_backward: poisoned in place on misuse
                 ctx.save_for_backward(d_h)
             else:
-                d_h, d_w = prepared.forward_backward(None, value)
+                d_h, d_w = prepared.forward_backward(None, value, dw_dtype)
                 ctx.save_for_backward(d_h, d_w)
             ctx.shapes = (hidden.shape, hidden.dtype, lm_head.dtype)
             if value is not None:
