@@ -68,6 +68,14 @@ def test_bad_descriptors(lib, kw, code):
     assert e.value.code == code and len(str(e.value)) > 20
 
 
+def test_every_documented_flag_is_accepted(lib):
+    assert (lib.FLAG_DW_ACCUMULATE, lib.FLAG_SFT, lib.FLAG_SKIP_MASKED, lib.FLAG_DW_BF16) == (1, 2, 4, 8)
+    base = lib.workspace_bytes(_desc(lib))
+    for flags in (lib.FLAG_DW_ACCUMULATE, lib.FLAG_SFT, lib.FLAG_DW_BF16, lib.FLAG_DW_ACCUMULATE | lib.FLAG_DW_BF16):
+        assert lib.workspace_bytes(_desc(lib, flags=flags)) == base      # none of these needs workspace
+    assert lib.workspace_bytes(_desc(lib, flags=lib.FLAG_SKIP_MASKED | lib.FLAG_DW_BF16))[1] > base[1]
+
+
 def test_null_and_workspace_errors_before_any_launch(lib):
     h = lib.load()
     d = _desc(lib)
