@@ -163,6 +163,68 @@ def _mfma_probe(torch, _lib, dev):
     return res
 
 
+def _neighbours(torch, M, _lib, cfg, wl, dev, iters=20) -> dict:
+    """The steps either side of the loss at this config's shape, each called through the C ABI and
+    timed with events on the stream it is launched on: final RMSNorm forward / backward
+    (llama/llama.py:426-452), the sampler's last-position logits and top-k draw
+    (sample_state_right_padding2.py:229-230, sanple_utils.py:35-53), the critic's value head
+    (plugins/training/ppo/module.py:34-52) and group advantages (advantage/grpo.py:28-52).  All but
+    the last are bound by HBM; `bytes` is the algorithmic traffic of one call."""
+    lib = _lib.load()
+    st = torch.cuda.current_stream(dev).cuda_stream
+    n, h, v = cfg.tokens, cfg.hidden, cfg.vocab
+    b_seq = wl["seq_shape"][0]
+    x, w = wl["hidden"], wl["lm_head"]
+    f32 = dict(dtype=torch.float32, device=dev)
+    scale = torch.ones(h, **f32)
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    rstd, dscale = torch.empty(n, **f32), torch.empty(h, **f32)
+    need = _lib.C.c_size_t(0)
+    _lib.check(lib.mj_rmsnorm_workspace_bytes(n, h, _lib.C.byref(need)))
+    nws = torch.empty(max(need.value, 16), dtype=torch.uint8, device=dev)
+    last = x[:: n // b_seq][:b_seq].contiguous()
+    logits = torch.empty((b_seq, v), **f32)
+    noise = torch.zeros((b_seq, 50), **f32)
+    token = torch.empty(b_seq, dtype=torch.int32, device=dev)
+    wv, bv, values = torch.full((h,), 0.01, **f32), torch.zeros(1, **f32), torch.empty(n, **f32)
+    rewards = torch.rand(b_seq, **f32)
+    gid = (torch.arange(b_seq, device=dev) // max(cfg.group, 1)).to(torch.int32)
+    adv = torch.empty(b_seq, **f32)
+    calls = {
+        "rmsnorm_forward": (lambda: lib.mj_rmsnorm_forward(x.data_ptr(), x.stride(0), scale.data_ptr(), y.data_ptr(), h,
+                                                          rstd.data_ptr(), n, h, 1e-6, st), 2 * n * h * 2 + n * 4),
+        "rmsnorm_backward": (lambda: lib.mj_rmsnorm_backward(y.data_ptr(), h, x.data_ptr(), x.stride(0), scale.data_ptr(),
+                                                            dx.data_ptr(), h, dscale.data_ptr(), 0, n, h, 1e-6,
+                                                            nws.data_ptr(), nws.numel(), st), 3 * n * h * 2),
+        "sample_logits": (lambda: lib.mj_sample_logits(last.data_ptr(), h, w.data_ptr(), w.stride(0), logits.data_ptr(), v,
+                                                      b_seq, h, v, float(cfg.softcap or 0.0), st),
+                          h * v * 2 + b_seq * h * 2 + b_seq * v * 4),
+        "sample_top_k": (lambda: lib.mj_sample_top_k(logits.data_ptr(), v, b_seq, v, 50, 1.0, noise.data_ptr(),
+                                                    token.data_ptr(), None, None, st), b_seq * v * 4),
+        "value_head_forward": (lambda: lib.mj_value_head_forward(x.data_ptr(), x.stride(0), wv.data_ptr(), bv.data_ptr(),
+                                                                values.data_ptr(), n, h, st), n * h * 2 + n * 4),
+        "group_advantages": (lambda: lib.mj_grpo_group_advantages(rewards.data_ptr(), gid.data_ptr(), adv.data_ptr(), b_seq,
+                                                                 1e-4, st), b_seq * 12),
+    }
+    rows = {}
+    for name, (fn, nbytes) in calls.items():
+        for _ in range(3):
+            _lib.check(fn())
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(iters):
+            _lib.check(fn())
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / iters
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        rows[name] = {"ms": round(ms, 4), "bytes": nbytes, "GB_per_s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / 8000.0, 4)}
+    return {"metric": "neighbour_steps", "config": {"workload": f"BASELINE configs shape {n} tokens x hidden {h} x vocab {v}",
+                                                    "sequences": b_seq}, "iters": iters,
+            "hbm_peak_GB_per_s": 8000.0, "rows": rows}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -186,6 +248,9 @@ def main() -> int:
                          "kernels + the in-place dZ pass instead of the default path")
     ap.add_argument("--dw-dtype", choices=("f32", "bf16"), default="f32",
                     help="dtype of the lm_head gradient the dW kernel writes (the reference's is float32: the default)")
+    ap.add_argument("--neighbours", action="store_true",
+                    help="instead of the loss step, time the steps either side of it (RMSNorm, sampler, value head, "
+                         "group advantages) at the config's shape against the HBM roofline")
     ap.add_argument("--no-kernel-events", action="store_true",
                     help="time the steps without the per-kernel HIP events (each event pair leaves ~10 us between "
                          "two kernels: nothing at the headline shape, 10 %% of a step at the smallest); the per-kernel "
@@ -246,6 +311,9 @@ def main() -> int:
             total_valid_token_count=wl["total_valid_token_count"], seq_shape=wl["seq_shape"],
             return_token_entropy=cfg.token_entropy, skip_masked=skip_masked, **step_kw, **kw)
 
+    if args.neighbours:
+        print(json.dumps(_neighbours(torch, M, _lib, cfg, wl, dev)), flush=True)
+        return 0
     if args.zero_operands:
         wl["hidden"].zero_()
         wl["lm_head"].zero_()

@@ -1149,17 +1149,92 @@ MJ_DEV float topk_unkey(uint32_t key) {
 constexpr int kTopKPool = 4096;
 
 __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
-  __shared__ uint32_t hist[4096];
+  __shared__ __attribute__((aligned(16))) uint32_t hist[4096];
+  uint64_t* ranked_word = (uint64_t*)hist;      // the common path's pool; the histogram paths start by clearing hist
   __shared__ uint32_t pool_key[kTopKPool];
   __shared__ int pool_idx[kTopKPool];
   __shared__ uint32_t s_scan[1024];
   __shared__ uint32_t s_prefix, s_need, s_cnt, s_pool, s_wave[16], s_base;
+  __shared__ float s_gmax[64];
   __shared__ float c_val[kTopKMax], o_val[kTopKMax];
   __shared__ int c_idx[kTopKMax], o_idx[kTopKMax];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* row = p.logits + (int64_t)blockIdx.x * p.ld;
 
-  // ---- fast path, two reads of the row: a 12-bit histogram finds the bin of the k-th largest
+  // Walks the row once, 16 bytes per lane where the row's address allows it, eight loads in flight
+  // per lane (the row comes from L2 or beyond: latency, not bandwidth, is what one workgroup sees).
+  const int v4 = (((uintptr_t)row & 15) == 0) ? (p.V & ~3) : 0;
+  auto for_each = [&](auto&& f) {
+    constexpr int U = 8;
+    int i = tid * 4;
+    for (; i + (U - 1) * 4096 < v4; i += U * 4096) {
+      f32x4 x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = *(const f32x4*)(row + i + u * 4096);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int j = i + u * 4096;
+        f(j, x[u][0]); f(j + 1, x[u][1]); f(j + 2, x[u][2]); f(j + 3, x[u][3]);
+      }
+    }
+    for (; i < v4; i += 4096) {
+      const f32x4 x = *(const f32x4*)(row + i);
+      f(i, x[0]); f(i + 1, x[1]); f(i + 2, x[2]); f(i + 3, x[3]);
+    }
+    for (int j = v4 + tid; j < p.V; j += 1024) f(j, row[j]);
+  };
+
+  // ---- common case, two reads of the row, no histogram and no division per element.  Threshold:
+  // the 1024 threads form 64 groups of 16 lanes; each group's largest logit belongs to some element,
+  // so at least 64 >= k elements reach the smallest of the 64 group maxima, `tau` (a group without
+  // elements or with nothing but NaNs leaves tau = -inf, and then every element qualifies).
+  // x -> key(x / t) is non-decreasing, so the k-th largest key is at least key(tau / t), and an
+  // element whose key reaches it has x >= tau up to the rounding of the two quotients: x >= tau_lo,
+  // a few ulps below tau.  Second read: elements that are not below tau_lo (NaNs included: their key
+  // is the largest) go to a pool with their exact keys -- a few hundred for logits of a language
+  // model -- where each one's rank under (key descending, index ascending) is counted directly.
+  // A pool that overflows (rows of near-equal values) takes the histogram paths below instead.
+  constexpr int kRankPool = 1024;
+  if (tid == 0) s_pool = 0;
+  float mx = -__builtin_inff();
+  for_each([&](int, float x) { mx = fmaxf(mx, x); });
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+  if ((lane & 15) == 0) s_gmax[wave * 4 + (lane >> 4)] = mx;
+  __syncthreads();
+  float tau = s_gmax[lane];
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) tau = fminf(tau, __shfl_xor(tau, o));
+  const float tau_lo = tau - fmaxf(fabsf(tau) * 0x1p-20f, 0x1p-100f);
+  for_each([&](int i, float x) {
+    if (!(x < tau_lo)) {
+      const uint32_t slot = atomicAdd(&s_pool, 1u);
+      // one 64-bit word per element whose order is (key descending, index ascending); never 0
+      if (slot < (uint32_t)kRankPool) ranked_word[slot] = ((uint64_t)topk_key(x / p.t) << 32) | (uint32_t)~i;
+    }
+  });
+  __syncthreads();
+  const uint32_t ranked = s_pool;
+  __syncthreads();                       // every thread has read s_pool before the paths below reset it
+  if (ranked <= (uint32_t)kRankPool) {
+    const uint32_t padded = (ranked + 7u) & ~7u;              // zeros behind the pool: smaller than any word
+    if ((uint32_t)tid >= ranked && (uint32_t)tid < padded) ranked_word[tid] = 0;
+    __syncthreads();
+    if ((uint32_t)tid < ranked) {
+      const uint64_t mine = ranked_word[tid];
+      int rank = 0;
+      for (uint32_t r = 0; r < padded; r += 8) {              // eight LDS reads in flight, not one
+        uint64_t w[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = ranked_word[r + j];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) rank += w[j] > mine ? 1 : 0;
+      }
+      if (rank < p.k) { c_val[rank] = topk_unkey((uint32_t)(mine >> 32)); c_idx[rank] = (int)~(uint32_t)mine; }
+    }
+    __syncthreads();
+  } else {
+  // ---- two reads of the row with a 12-bit histogram: finds the bin of the k-th largest
   // key; a second read sends larger keys straight to the result and the bin's keys to an LDS pool,
   // where the selection finishes.  A bin that overflows the pool (many near-equal logits) falls
   // back to the byte-wise select below.
@@ -1329,14 +1404,16 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
     __syncthreads();
   }
   }
+  }
   // order the k candidates: value descending, index ascending
   if (tid < p.k) {
     const float v = c_val[tid];
     const int ix = c_idx[tid];
     int r = 0;
-    for (int j = 0; j < p.k; ++j) {
+#pragma unroll 16
+    for (int j = 0; j < kTopKMax; ++j) {       // fixed trip count: the LDS reads go out in batches
       const float vj = c_val[j];
-      r += (vj > v || (vj == v && c_idx[j] < ix)) ? 1 : 0;
+      r += (j < p.k && (vj > v || (vj == v && c_idx[j] < ix))) ? 1 : 0;
     }
     o_val[r] = v;
     o_idx[r] = ix;
@@ -1345,15 +1422,20 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
   if (tid < p.k) {
     if (p.top_idx != nullptr) p.top_idx[(int64_t)blockIdx.x * p.k + tid] = o_idx[tid];
     if (p.top_val != nullptr) p.top_val[(int64_t)blockIdx.x * p.k + tid] = o_val[tid];
+    // the k noise values in one go (c_val is free again): the scan below then stays inside the LDS
+    if (p.noise != nullptr) c_val[tid] = o_val[tid] + p.noise[(int64_t)blockIdx.x * p.k + tid];
   }
+  __syncthreads();
   if (tid == 0) {
     int best = 0;
     if (p.noise != nullptr) {
-      float bs = o_val[0] + p.noise[(int64_t)blockIdx.x * p.k];
-      for (int j = 1; j < p.k; ++j) {
-        const float sc = o_val[j] + p.noise[(int64_t)blockIdx.x * p.k + j];
-        if (sc > bs) { bs = sc; best = j; }      // first maximum wins, like argmax
-      }
+      float sc[kTopKMax];
+#pragma unroll
+      for (int j = 0; j < kTopKMax; ++j) sc[j] = c_val[j];
+      float bs = sc[0];
+#pragma unroll
+      for (int j = 1; j < kTopKMax; ++j)
+        if (j < p.k && sc[j] > bs) { bs = sc[j]; best = j; }      // first maximum wins, like argmax
     }
     p.token[blockIdx.x] = o_idx[best];
   }
