@@ -206,6 +206,10 @@ def _neighbours(torch, M, _lib, cfg, wl, dev, iters=20) -> dict:
         "group_advantages": (lambda: lib.mj_grpo_group_advantages(rewards.data_ptr(), gid.data_ptr(), adv.data_ptr(), b_seq,
                                                                  1e-4, st), b_seq * 12),
     }
+    def vendor_product():       # the same product through torch.matmul (hipBLASLt), bf16 result: a yardstick only
+        torch.matmul(last, w)
+        return 0
+    calls["vendor_matmul_for_sample_logits"] = (vendor_product, h * v * 2 + b_seq * h * 2 + b_seq * v * 2)
     rows = {}
     for name, (fn, nbytes) in calls.items():
         for _ in range(3):

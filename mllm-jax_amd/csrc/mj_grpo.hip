@@ -723,12 +723,34 @@ int mj_sample_logits(const void* hidden, int64_t ld_hidden, const void* lm_head,
   if (ld_w > (1 << 21) || ld_logits > (1 << 21) || ld_hidden > (1 << 20))
     return fail(MJ_GRPO_ERR_SHAPE, "sample_logits: leading dimensions too large (ld_hidden <= 2^20; ld_w, ld_logits <= 2^21)");
   int rc;
-  if ((rc = enable_lds(mj::k_logits_rows<BM, BN>))) return rc;
   mj::LogitsRowsArgs a;
   a.w = (const __bf16*)lm_head; a.hid = (const __bf16*)hidden; a.ld_w = ld_w; a.ld_hid = ld_hidden;
   a.V = (int)vocab; a.n = (int)b; a.H = (int)h; a.cap = softcap; a.out = logits; a.ld_out = ld_logits;
-  const mj::TileMap map = mj::TileMap::pick_shape((int)((vocab + BM - 1) / BM), (int)((b + BN - 1) / BN), 1, 1);
-  mj::k_logits_rows<BM, BN><<<map.items(), mj::kThreads, mj::GemmTN<BM, BN>::kLdsBytes, (hipStream_t)stream>>>(a, map);
+  // Batch-row tile and vocab columns per work item: the fewest rounds of resident workgroups (one
+  // per CU; two with the 64-row tile, whose LDS stages are 80 KB) whose items are <= 256 columns wide.
+  const int bn = b <= 64 ? 64 : b <= 128 ? 128 : 256;
+  const int64_t tiles_n = (b + bn - 1) / bn;
+  const int64_t slots = 256 * (bn == 64 ? 2 : 1);
+  int64_t tile_rows = BM;
+  for (int64_t rounds = 1; rounds <= 4096; ++rounds) {
+    const int64_t per = slots * rounds / tiles_n;            // items along the vocabulary
+    if (per == 0) continue;
+    const int64_t cols = rup((vocab + per - 1) / per, 8);
+    if (cols <= BM) { tile_rows = cols; break; }
+  }
+  a.tile_rows = (int)tile_rows;
+  const mj::TileMap map = mj::TileMap::pick_shape((int)((vocab + tile_rows - 1) / tile_rows), (int)tiles_n, 1, 1);
+  hipStream_t st = (hipStream_t)stream;
+  if (bn == 64) {
+    if ((rc = enable_lds(mj::k_logits_rows<BM, 64>))) return rc;
+    mj::k_logits_rows<BM, 64><<<map.items(), mj::kThreads, mj::GemmTN<BM, 64>::kLdsBytes, st>>>(a, map);
+  } else if (bn == 128) {
+    if ((rc = enable_lds(mj::k_logits_rows<BM, 128>))) return rc;
+    mj::k_logits_rows<BM, 128><<<map.items(), mj::kThreads, mj::GemmTN<BM, 128>::kLdsBytes, st>>>(a, map);
+  } else {
+    if ((rc = enable_lds(mj::k_logits_rows<BM, BN>))) return rc;
+    mj::k_logits_rows<BM, BN><<<map.items(), mj::kThreads, mj::GemmTN<BM, BN>::kLdsBytes, st>>>(a, map);
+  }
   return check_launch("k_logits_rows");
 }
 
@@ -836,3 +858,5 @@ template __global__ void mj::k_dhidden<256, 256>(mj::DhArgs, mj::TileMap);
 template __global__ void mj::k_dw<256, 256, false>(mj::DwArgs, mj::TileMap);
 template __global__ void mj::k_dw<256, 256, true>(mj::DwArgs, mj::TileMap);
 template __global__ void mj::k_logits_rows<256, 256>(mj::LogitsRowsArgs, mj::TileMap);
+template __global__ void mj::k_logits_rows<256, 128>(mj::LogitsRowsArgs, mj::TileMap);
+template __global__ void mj::k_logits_rows<256, 64>(mj::LogitsRowsArgs, mj::TileMap);

@@ -1081,17 +1081,24 @@ struct LogitsRowsArgs {
   float cap;             // final-logit softcap, 0 = off
   float* out;            // [n, ld_out]
   int64_t ld_out;
+  int tile_rows;         // vocab columns per work item: a multiple of 8, <= BM
 };
 
+// A decode batch is a few rows against the whole vocabulary matrix: the product is bound by reading
+// W once.  BN follows the batch (64 / 128 / 256 rows, so the MFMA work per slice does not outlast
+// its loads) and a work item covers `tile_rows` <= BM vocab columns, chosen on the host so that the
+// items fill whole rounds of the resident workgroups; the columns of the 256-wide tile past
+// tile_rows are neither loaded (the operand's row limit) nor stored.
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void k_logits_rows(LogitsRowsArgs p, TileMap map) {
-  using G = GemmTN<BM, BN, kKRow, kRowK>;
+  using G = GemmTN<BM, BN, kKRow, kRowK, (BN < 256 ? 2 : 1)>;   // the narrow tiles wait on memory: three slices in flight
   extern __shared__ __attribute__((aligned(16))) char smem[];
   int tm, tn, split;
   if (!map.tile(blockIdx.x, tm, tn, split)) return;
-  const int m0 = tm * BM, n0 = tn * BN;
+  const int m0 = tm * p.tile_rows, n0 = tn * BN;
+  const int m1 = min(p.V, m0 + p.tile_rows);
   G g;
-  g.run(p.w + m0, p.V - m0, p.ld_w, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0, p.ld_hid, p.H, smem);
+  g.run(p.w + m0, m1 - m0, p.ld_w, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0, p.ld_hid, p.H, smem);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
@@ -1099,7 +1106,7 @@ __global__ __launch_bounds__(kThreads) void k_logits_rows(LogitsRowsArgs p, Tile
   const int trows = min(max(p.n - t0, 0), G::WN);
   const uint32_t ld4 = (uint32_t)p.ld_out * 4;
   const __amdgpu_buffer_rsrc_t rs = make_rsrc_wave(p.out + (int64_t)t0 * p.ld_out + v0, (int64_t)trows * ld4 - (int64_t)v0 * 4);
-  const int vleft = p.V - v0;
+  const int vleft = m1 - v0;             // columns of this work item from the wavefront's first on (may be <= 0)
   const float inv_cap = p.cap > 0.f ? 1.f / p.cap : 0.f;
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {

@@ -13,7 +13,11 @@ def test_last_position_logits_match_float64_product():
     import mllm_jax_amd as M
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(1)
-    for b, h, v, cap in [(5, 64, 1000, None), (128, 896, 5000, None), (300, 136, 2008, 30.0), (1, 8, 8, None)]:
+    # batch sizes either side of the 64- and 128-row tiles, vocabularies that give work items of
+    # 8 .. 256 columns, one full-size vocabulary
+    for b, h, v, cap in [(5, 64, 1000, None), (128, 896, 5000, None), (300, 136, 2008, 30.0), (1, 8, 8, None),
+                         (64, 72, 3000, None), (65, 72, 3000, None), (129, 64, 1000, 10.0), (16, 128, 152064, None),
+                         (100, 64, 66000, None)]:
         hid = torch.randn(b, h, generator=g).to(torch.bfloat16)
         w = (0.2 * torch.randn(h, v, generator=g)).to(torch.bfloat16)
         out = M.last_position_logits(hid.to(dev), w.to(dev), cap)
@@ -33,6 +37,36 @@ def test_top_k_draw_is_bit_exact(b, v, k, t):
     noise = -torch.log(-torch.log(u))
     tok, idx, val = M.top_k_sampling_batched(noise.to(dev), logits.to(dev), k=k, t=t, return_top_k=True)
     rt, ri, rv = O.top_k_sample(logits.numpy(), k=k, t=t, noise=noise.numpy())
+    np.testing.assert_array_equal(idx.cpu().numpy(), ri)
+    np.testing.assert_array_equal(val.cpu().numpy(), rv)
+    np.testing.assert_array_equal(tok.cpu().numpy(), rt)
+
+
+@pytest.mark.parametrize("t", [3.0, 1.7, 0.6])
+def test_neighbouring_floats_that_divide_to_the_same_quotient(t):
+    """A cluster of adjacent float32 values around the k-th largest: after the division by t > 1
+    neighbours collapse into equal quotients and the lower index must win, also for elements that
+    sit a few ulps below the kernel's raw-value threshold."""
+    import mllm_jax_amd as M
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(7)
+    b, v, k = 4, 70000, 50
+    x = rng.normal(-5.0, 0.5, size=(b, v)).astype(np.float32)
+    for r in range(b):
+        pos = rng.choice(v, size=300, replace=False)
+        steps = rng.integers(0, 40, size=300)
+        base = np.float32([2.0, -1.5, 1e-3, 300.0][r])
+        vals = base.copy()
+        cluster = np.array([np.nextafter(base, np.float32(np.inf), dtype=np.float32)] * 300, np.float32)
+        for j, s_ in enumerate(steps):
+            c = base
+            for _ in range(int(s_)):
+                c = np.nextafter(c, np.float32(np.inf), dtype=np.float32)
+            cluster[j] = c
+        x[r, pos] = cluster
+    noise = rng.gumbel(size=(b, k)).astype(np.float32)
+    tok, idx, val = M.top_k_sampling_batched(torch.tensor(noise), torch.tensor(x, device=dev), k=k, t=t, return_top_k=True)
+    rt, ri, rv = O.top_k_sample(x, k=k, t=t, noise=noise)
     np.testing.assert_array_equal(idx.cpu().numpy(), ri)
     np.testing.assert_array_equal(val.cpu().numpy(), rv)
     np.testing.assert_array_equal(tok.cpu().numpy(), rt)
