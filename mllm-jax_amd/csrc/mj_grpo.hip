@@ -773,9 +773,8 @@ int mj_sample_top_k(const float* logits, int64_t ld_logits, int64_t b, int64_t v
 // ----------------------------------------------------------------------------- RMSNorm
 namespace {
 constexpr int kNormMaxH = 8192;
-int norm_grid(int64_t n) {   // workgroups of the backward: enough to fill the GPU, each walks rows with this stride
-  const int64_t blocks = (n + 3) / 4;
-  return (int)(blocks < 512 ? blocks : 512);
+int norm_grid(int64_t n) {   // workgroups of the backward (one row at a time each, rows with this stride): four per CU
+  return (int)(n < 1024 ? n : 1024);
 }
 int norm_check(int64_t n, int64_t h, std::initializer_list<int64_t> lds, std::initializer_list<const void*> ptrs) {
   if (n <= 0 || h <= 0 || n > (1ll << 30)) return fail(MJ_GRPO_ERR_SHAPE, "rmsnorm: n and h must be positive (got %lld, %lld)", (long long)n, (long long)h);
@@ -820,27 +819,17 @@ int mj_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x, int64_t ld
   int rc = norm_check(n, h, {ld_dy, ld_x, ld_dx}, {dy, x, scale, dx, workspace});
   if (rc) return rc;
   if (dscale == nullptr) return fail(MJ_GRPO_ERR_NULL, "rmsnorm: dscale is NULL");
+  if (misaligned(dscale)) return fail(MJ_GRPO_ERR_ALIGN, "rmsnorm: pointers must be 16-byte aligned");
   const int grid = norm_grid(n);
   const size_t need = (size_t)grid * (size_t)h * 4;
   if (workspace_bytes < need) return fail(MJ_GRPO_ERR_WORKSPACE, "rmsnorm: workspace too small: %zu < %zu bytes", workspace_bytes, need);
   mj::NormBwdArgs a;
   a.dy = (const uint16_t*)dy; a.x = (const uint16_t*)x; a.scale = scale; a.dx = (uint16_t*)dx;
   a.part = (float*)workspace; a.ld_dy = ld_dy; a.ld_x = ld_x; a.ld_dx = ld_dx; a.n = (int)n; a.H = (int)h; a.eps = eps;
-  const size_t lds = 3 * (size_t)h * 4;
   hipStream_t st = (hipStream_t)stream;
-  if (h <= 4096) {
-    mj::k_rmsnorm_bwd<8><<<grid, 256, lds, st>>>(a);
-  } else {
-    static thread_local int raised_dev = -1;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipGetDevice failed");
-    if (raised_dev != dev) {
-      hipError_t e = hipFuncSetAttribute((const void*)mj::k_rmsnorm_bwd<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * kNormMaxH * 4);
-      if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-      raised_dev = dev;
-    }
-    mj::k_rmsnorm_bwd<16><<<grid, 256, lds, st>>>(a);
-  }
+  if (h <= 2048) mj::k_rmsnorm_bwd<1><<<grid, 256, 0, st>>>(a);
+  else if (h <= 4096) mj::k_rmsnorm_bwd<2><<<grid, 256, 0, st>>>(a);
+  else mj::k_rmsnorm_bwd<4><<<grid, 256, 0, st>>>(a);
   if ((rc = check_launch("k_rmsnorm_bwd"))) return rc;
   mj::k_rmsnorm_dscale<<<(unsigned)((h + 63) / 64), 256, 0, st>>>((const float*)workspace, grid, (int)h, dscale,
                                                                   accumulate_dscale);

@@ -125,8 +125,8 @@ def test_rmsnorm_argument_checks_before_any_launch(lib):
     h = lib.load()
     fake = 0x1000   # never dereferenced: argument checks fail first
     sz = C.c_size_t()
-    assert h.mj_rmsnorm_workspace_bytes(4096, 3584, C.byref(sz)) == 0 and sz.value == 512 * 3584 * 4
-    assert h.mj_rmsnorm_workspace_bytes(10, 64, C.byref(sz)) == 0 and sz.value == 3 * 64 * 4
+    assert h.mj_rmsnorm_workspace_bytes(4096, 3584, C.byref(sz)) == 0 and sz.value == 1024 * 3584 * 4
+    assert h.mj_rmsnorm_workspace_bytes(10, 64, C.byref(sz)) == 0 and sz.value == 10 * 64 * 4     # one partial row per workgroup, one workgroup per row up to 1024
     assert h.mj_rmsnorm_workspace_bytes(0, 64, C.byref(sz)) == 2
     assert h.mj_rmsnorm_workspace_bytes(8, 60, C.byref(sz)) == 3
     assert h.mj_rmsnorm_workspace_bytes(8, 16384, C.byref(sz)) == 5 and b"8192" in h.mj_grpo_last_error()
