@@ -727,10 +727,12 @@ int mj_sample_logits(const void* hidden, int64_t ld_hidden, const void* lm_head,
   a.w = (const __bf16*)lm_head; a.hid = (const __bf16*)hidden; a.ld_w = ld_w; a.ld_hid = ld_hidden;
   a.V = (int)vocab; a.n = (int)b; a.H = (int)h; a.cap = softcap; a.out = logits; a.ld_out = ld_logits;
   // Batch-row tile and vocab columns per work item: the fewest rounds of resident workgroups (one
-  // per CU; two with the 64-row tile, whose LDS stages are 80 KB) whose items are <= 256 columns wide.
-  const int bn = b <= 64 ? 64 : b <= 128 ? 128 : 256;
+  // per CU) whose items are <= 256 columns wide.  Measured at 3584 x 152064: the 128-row tile beats
+  // both a 64-row tile with two workgroups per CU (0.25 against 0.23 ms at 64 rows) and, past 128
+  // rows, is beaten by the 256-row tile (two 128-row tiles: 0.35 against 0.32 ms at 192 rows).
+  const int bn = b <= 128 ? 128 : 256;
   const int64_t tiles_n = (b + bn - 1) / bn;
-  const int64_t slots = 256 * (bn == 64 ? 2 : 1);
+  const int64_t slots = 256;
   int64_t tile_rows = BM;
   for (int64_t rounds = 1; rounds <= 4096; ++rounds) {
     const int64_t per = slots * rounds / tiles_n;            // items along the vocabulary
@@ -741,10 +743,7 @@ int mj_sample_logits(const void* hidden, int64_t ld_hidden, const void* lm_head,
   a.tile_rows = (int)tile_rows;
   const mj::TileMap map = mj::TileMap::pick_shape((int)((vocab + tile_rows - 1) / tile_rows), (int)tiles_n, 1, 1);
   hipStream_t st = (hipStream_t)stream;
-  if (bn == 64) {
-    if ((rc = enable_lds(mj::k_logits_rows<BM, 64>))) return rc;
-    mj::k_logits_rows<BM, 64><<<map.items(), mj::kThreads, mj::GemmTN<BM, 64>::kLdsBytes, st>>>(a, map);
-  } else if (bn == 128) {
+  if (bn == 128) {
     if ((rc = enable_lds(mj::k_logits_rows<BM, 128>))) return rc;
     mj::k_logits_rows<BM, 128><<<map.items(), mj::kThreads, mj::GemmTN<BM, 128>::kLdsBytes, st>>>(a, map);
   } else {
@@ -848,4 +847,3 @@ template __global__ void mj::k_dw<256, 256, false>(mj::DwArgs, mj::TileMap);
 template __global__ void mj::k_dw<256, 256, true>(mj::DwArgs, mj::TileMap);
 template __global__ void mj::k_logits_rows<256, 256>(mj::LogitsRowsArgs, mj::TileMap);
 template __global__ void mj::k_logits_rows<256, 128>(mj::LogitsRowsArgs, mj::TileMap);
-template __global__ void mj::k_logits_rows<256, 64>(mj::LogitsRowsArgs, mj::TileMap);

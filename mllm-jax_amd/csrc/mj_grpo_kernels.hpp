@@ -1085,8 +1085,8 @@ struct LogitsRowsArgs {
 };
 
 // A decode batch is a few rows against the whole vocabulary matrix: the product is bound by reading
-// W once.  BN follows the batch (64 / 128 / 256 rows, so the MFMA work per slice does not outlast
-// its loads) and a work item covers `tile_rows` <= BM vocab columns, chosen on the host so that the
+// W once.  BN follows the batch (128 or 256 rows, so the MFMA work per slice does not outlast its
+// loads) and a work item covers `tile_rows` <= BM vocab columns, chosen on the host so that the
 // items fill whole rounds of the resident workgroups; the columns of the 256-wide tile past
 // tile_rows are neither loaded (the operand's row limit) nor stored.
 template <int BM, int BN>

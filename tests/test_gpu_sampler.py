@@ -13,7 +13,7 @@ def test_last_position_logits_match_float64_product():
     import mllm_jax_amd as M
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(1)
-    # batch sizes either side of the 64- and 128-row tiles, vocabularies that give work items of
+    # batch sizes either side of the 128-row tile, vocabularies that give work items of
     # 8 .. 256 columns, one full-size vocabulary
     for b, h, v, cap in [(5, 64, 1000, None), (128, 896, 5000, None), (300, 136, 2008, 30.0), (1, 8, 8, None),
                          (64, 72, 3000, None), (65, 72, 3000, None), (129, 64, 1000, 10.0), (16, 128, 152064, None),
