@@ -102,3 +102,30 @@ def test_other_gradient_dtypes_are_refused():
     args, _ = _inputs(59)
     with pytest.raises(ValueError, match="float32 or bfloat16"):
         M.grpo_loss_value_and_grad(*args, lm_head_grad_dtype=torch.float16)
+
+
+def test_separate_backward_writes_the_rounded_float32_gradient():
+    """mj_grpo_backward (the transpose pass alone, from saved lse / logp) with the flag set."""
+    import ctypes as C
+    from mllm_jax_amd import _lib
+    from mllm_jax_amd.loss import _Prepared, _workspace, _ptr
+    args, ref = _inputs(61)
+    kw = dict(total_valid_token_count=None, epsilon_low=0.2, epsilon_high=0.3, temperature=1.0,
+              final_logit_softcap=None, seq_shape=None, chunk_tokens=1024)
+    p = _Prepared(*args, **kw)
+    p.forward()
+    _, both = _lib.workspace_bytes(p.desc)
+    ws = _workspace(args[0].device, both)
+    out = {}
+    for name, dtype, flag in (("f32", torch.float32, 0), ("bf16", torch.bfloat16, _lib.FLAG_DW_BF16)):
+        dh = torch.empty((N, H), dtype=torch.bfloat16, device=ws.device)
+        dw = torch.empty((H, V), dtype=dtype, device=ws.device)
+        p.desc.flags = flag
+        _lib.check(_lib.load().mj_grpo_backward(
+            C.byref(p.desc), _ptr(p.hidden), _ptr(p.w), _ptr(p.targets), _ptr(p.old), _ptr(p.adv), _ptr(p.mask),
+            _ptr(p.lse), _ptr(p.logp), _ptr(dh), _ptr(dw), _ptr(ws), ws.numel(), p.stream()))
+        torch.cuda.synchronize()
+        out[name] = (dh, dw)
+    assert torch.equal(out["bf16"][1], out["f32"][1].to(torch.bfloat16))
+    assert torch.equal(out["bf16"][0], out["f32"][0])
+    assert _rel(out["bf16"][1].float().cpu().numpy(), ref["d_lm_head"]) <= GRAD_RTOL
