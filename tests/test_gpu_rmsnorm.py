@@ -15,7 +15,8 @@ def _rel(a, b):
     return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
 
 
-@pytest.mark.parametrize("n,h", [(1, 8), (7, 64), (300, 896), (1027, 3584), (64, 4096), (33, 4104), (16, 8192)])
+@pytest.mark.parametrize("n,h", [(1, 8), (7, 64), (300, 896), (1027, 3584), (64, 4096), (33, 4104), (16, 8192),
+                                 (2100, 2048), (5, 2056), (3000, 1536)])
 def test_forward_backward_match_oracle(n, h):
     import mllm_jax_amd as M
     dev = torch.device("cuda:0")
