@@ -246,12 +246,18 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
   int* state = (int*)(ws + p.state);
   float* rs = (float*)(ws + p.rs);
   uint16_t* hs = (uint16_t*)(ws + p.hs);
+  // the logits kernels exist with and without the softcap code (a template parameter)
+  const bool cap = d->softcap > 0.f;
+  auto k_grad = cap ? mj::k_logits_stats<BM, BN, mj::kStatsGrad, false, true> : mj::k_logits_stats<BM, BN, mj::kStatsGrad, false, false>;
+  auto k_exp = cap ? mj::k_logits_stats<BM, BN, mj::kStatsExp, false, true> : mj::k_logits_stats<BM, BN, mj::kStatsExp, false, false>;
+  auto k_max = cap ? mj::k_logits_stats<BM, BN, mj::kStatsMax, false, true> : mj::k_logits_stats<BM, BN, mj::kStatsMax, false, false>;
+  auto k_max_rescue = cap ? mj::k_logits_stats<BM, BN, mj::kStatsMax, true, true> : mj::k_logits_stats<BM, BN, mj::kStatsMax, true, false>;
   if (mode == kBackwardOnly) {
-    if ((rc = enable_lds(mj::k_logits_stats<BM, BN, mj::kStatsGrad, false>))) return rc;
+    if ((rc = enable_lds(k_grad))) return rc;
   } else {
-    if (exp_mode && (rc = enable_lds(mj::k_logits_stats<BM, BN, mj::kStatsExp, false>))) return rc;
-    if (exp_mode && (rc = enable_lds(mj::k_logits_stats<BM, BN, mj::kStatsMax, true>))) return rc;
-    if (!exp_mode && (rc = enable_lds(mj::k_logits_stats<BM, BN, mj::kStatsMax, false>))) return rc;
+    if (exp_mode && (rc = enable_lds(k_exp))) return rc;
+    if (exp_mode && (rc = enable_lds(k_max_rescue))) return rc;
+    if (!exp_mode && (rc = enable_lds(k_max))) return rc;
   }
   if (bwd) {
     if ((rc = enable_lds(mj::k_dhidden<BM, BN>))) return rc;
@@ -361,7 +367,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       a.lse = saved_lse + c0;
       {
         Timed t(MJ_GRPO_K_LOGITS_STATS, st);
-        mj::k_logits_stats<BM, BN, mj::kStatsGrad, false><<<map.items(), mj::kThreads, lds, st>>>(a, map);
+        k_grad<<<map.items(), mj::kThreads, lds, st>>>(a, map);
       }
       Timed t(MJ_GRPO_K_FINALIZE, st);
       mj::k_patch_grad<<<(nc + 255) / 256, 256, 0, st>>>(zt, p.ld_z, zy + c0, saved_lse + c0, g, targets + c0, nc, V,
@@ -369,7 +375,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     } else if (exp_mode) {
       {
         Timed t(MJ_GRPO_K_LOGITS_STATS, st);
-        mj::k_logits_stats<BM, BN, mj::kStatsExp, false><<<map.items(), mj::kThreads, lds, st>>>(a, map);
+        k_exp<<<map.items(), mj::kThreads, lds, st>>>(a, map);
       }
       {
         Timed t(MJ_GRPO_K_FINALIZE, st);
@@ -384,13 +390,13 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       // range check in k_finalize failed
       Timed t(MJ_GRPO_K_RESCUE, st);
       f.rescue = 1; z.rescue = 1;
-      mj::k_logits_stats<BM, BN, mj::kStatsMax, true><<<kRescueGrid, mj::kThreads, lds, st>>>(a, map);
+      k_max_rescue<<<kRescueGrid, mj::kThreads, lds, st>>>(a, map);
       mj::k_finalize<mj::kStatsMax><<<n_pad / mj::kFinTokens, mj::kFinTokens * mj::kFinSlices, 0, st>>>(f);
       if (bwd) mj::k_dz<<<dz_grid, 256, 0, st>>>(z);
     } else {
       {
         Timed t(MJ_GRPO_K_LOGITS_STATS, st);
-        mj::k_logits_stats<BM, BN, mj::kStatsMax, false><<<map.items(), mj::kThreads, lds, st>>>(a, map);
+        k_max<<<map.items(), mj::kThreads, lds, st>>>(a, map);
       }
       {
         Timed t(MJ_GRPO_K_FINALIZE, st);
@@ -838,10 +844,14 @@ int mj_rmsnorm_backward(const void* dy, int64_t ld_dy, const void* x, int64_t ld
 }  // extern "C"
 
 // Explicit instantiations of the tile kernels used above.
-template __global__ void mj::k_logits_stats<256, 256, mj::kStatsExp, false>(mj::LogitsArgs, mj::TileMap);
-template __global__ void mj::k_logits_stats<256, 256, mj::kStatsMax, false>(mj::LogitsArgs, mj::TileMap);
-template __global__ void mj::k_logits_stats<256, 256, mj::kStatsMax, true>(mj::LogitsArgs, mj::TileMap);
-template __global__ void mj::k_logits_stats<256, 256, mj::kStatsGrad, false>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsExp, false, false>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsExp, false, true>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsMax, false, false>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsMax, false, true>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsMax, true, false>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsMax, true, true>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsGrad, false, false>(mj::LogitsArgs, mj::TileMap);
+template __global__ void mj::k_logits_stats<256, 256, mj::kStatsGrad, false, true>(mj::LogitsArgs, mj::TileMap);
 template __global__ void mj::k_dhidden<256, 256>(mj::DhArgs, mj::TileMap);
 template __global__ void mj::k_dw<256, 256, false>(mj::DwArgs, mj::TileMap);
 template __global__ void mj::k_dw<256, 256, true>(mj::DwArgs, mj::TileMap);

@@ -147,7 +147,7 @@ MJ_DEV void store_rows8(const float (&v)[8], uint32_t keep, __amdgpu_buffer_rsrc
 }
 
 // One 256 x 256 tile: logits^T [vocab x tokens] = W^T * hidden^T on MFMA, then the epilogue of MODE.
-template <int BM, int BN, int MODE>
+template <int BM, int BN, int MODE, bool CAP>
 MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
   using G = GemmTN<BM, BN, kKRow, kRowK>;
   const int m0 = tm * BM, n0 = tn * BN;
@@ -161,7 +161,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
   const int vbase = vwave + lhi * 4;             // + mi*32 + (r/4)*8 + r%4
   const int t0 = n0 + wn * G::WN;                // first token of this wavefront
   const bool tail = (m0 + BM > p.V);
-  const float inv_cap = p.cap > 0.f ? 1.f / p.cap : 0.f;
+  const float inv_cap = CAP ? 1.f / p.cap : 0.f;
   const float inv_cap2 = inv_cap * inv_cap;
   const int zt_cols = live_pad(p.n_live, p.c0, (p.n + 255) & ~255);
   // this wavefront's 128 token rows of the 16-bit matrix; rows at or past n fall outside and are dropped
@@ -172,16 +172,32 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
     const int col = t0 + ni * 32 + l31;
-    // Softcap and the stand-in for rows past V are rare, wave-uniform cases: each sits behind a
-    // real scalar branch (the empty asm keeps the compiler from flattening it into per-element
-    // selects, which would cost an exp and a reciprocal per logit whether or not a cap is set).
-    if (p.cap > 0.f) {
-      asm volatile("");
+    // Softcap (CAP: a kernel of its own, so that the uncapped one carries none of this).  While every
+    // logit of the block is small against the cap -- checked per wavefront -- tanh is its odd series
+    // to u^7 (|u| <= 0.25: error below 1e-7 of u, five multiply-adds instead of an exp and a reciprocal).
+    if (CAP) {
+      float big = 0.f;
 #pragma unroll
       for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) g.acc[mi][ni][r] = softcap_apply(g.acc[mi][ni][r], p.cap, inv_cap);
+        for (int r = 0; r < 16; ++r) big = fmaxf(big, fabsf(g.acc[mi][ni][r]));
+      if (__all(big * inv_cap <= 0.25f)) {
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float z = g.acc[mi][ni][r], u = z * inv_cap, u2 = u * u;
+            g.acc[mi][ni][r] = z * fmaf(u2, fmaf(u2, fmaf(u2, -17.f / 315.f, 2.f / 15.f), -1.f / 3.f), 1.f);
+          }
+      } else {
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) g.acc[mi][ni][r] = softcap_apply(g.acc[mi][ni][r], p.cap, inv_cap);
+      }
     }
+    // The stand-in for rows past V is a rare, wave-uniform case behind a real scalar branch (the
+    // empty asm keeps the compiler from flattening it into per-element selects).
     if (tail) {
       asm volatile("");
 #pragma unroll
@@ -269,7 +285,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
               const float e = __builtin_amdgcn_exp2f(z * kLog2e);
               l += e;
               s = fmaf(e, z, s);
-              v[j] = p.cap > 0.f ? e * (1.f - z * z * inv_cap2) : e;
+              v[j] = CAP ? e * (1.f - z * z * inv_cap2) : e;
             }
             store_rows8<false>(v, keep, zrs, group_off(mi, qp), (uint32_t)(mi * 32 + qp * 16) * 2);
           }
@@ -304,7 +320,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
             for (int j = 0; j < 8; ++j) {
               const float z = g.acc[mi][ni][qp * 8 + j];
               const float d = gneg * __builtin_amdgcn_exp2f(fmaf(z, kLog2e, -lse2));
-              v[j] = p.cap > 0.f ? d * (1.f - z * z * inv_cap2) : d;
+              v[j] = CAP ? d * (1.f - z * z * inv_cap2) : d;
             }
             store_rows8<false>(v, gneg != 0.f ? 0xffffffffu : 0u, zrs, group_off(mi, qp),
                                (uint32_t)(mi * 32 + qp * 16) * 2);
@@ -332,20 +348,20 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
 
 // One workgroup per tile; RESCUE: a small grid that walks the tile list, and leaves at once unless
 // the range check of the kStatsExp pass failed (state != 0).
-template <int BM, int BN, int MODE, bool RESCUE>
+template <int BM, int BN, int MODE, bool RESCUE, bool CAP>
 __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap map) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   int tm, tn, split;
   if (RESCUE) {
     if (__builtin_amdgcn_readfirstlane(*p.state) == 0) return;
     for (int item = blockIdx.x; item < map.items(); item += gridDim.x) {
-      if (map.tile(item, tm, tn, split)) logits_tile<BM, BN, MODE>(p, tm, tn, smem);
+      if (map.tile(item, tm, tn, split)) logits_tile<BM, BN, MODE, CAP>(p, tm, tn, smem);
       __syncthreads();      // the next tile's first LDS writes must not pass this tile's last reads
     }
   } else {
     if (MODE == kStatsExp && blockIdx.x == 0 && threadIdx.x == 0) *p.state = 0;
     if (!map.tile(blockIdx.x, tm, tn, split)) return;
-    logits_tile<BM, BN, MODE>(p, tm, tn, smem);
+    logits_tile<BM, BN, MODE, CAP>(p, tm, tn, smem);
   }
 }
 
