@@ -470,7 +470,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
 
 extern "C" {
 
-int mj_grpo_version(void) { return 200; }
+int mj_grpo_version(void) { return 300; }   // 0.3.0: MJ_GRPO_FLAG_DW_BF16, d_lm_head as void*
 
 const char* mj_grpo_last_error(void) { return g_err; }
 
