@@ -330,6 +330,8 @@ def main() -> int:
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    if 64 * args.steps > 60000:          # more event pairs than the library's profiler takes (65536)
+        args.no_kernel_events = True
     if not args.no_kernel_events:
         _lib.profile_begin(64 * max(args.steps, 1))
     sampler = _SmiSampler() if args.smi else None
