@@ -1144,7 +1144,8 @@ __global__ __launch_bounds__(kThreads) void k_logits_rows(LogitsRowsArgs p, Tile
 }
 
 // Top-k + categorical draw per row (MLLM_JAX/sample/sanple_utils.py:35-53): the k largest of
-// logits / t (ties: lower index first, like jax.lax.top_k), then argmax_j(top_j + noise_j) where
+// logits / t in the IEEE total order (-0 below +0, NaN largest, as XLA's sort comparators order
+// floats; ties: lower index first, like jax.lax.top_k), then argmax_j(top_j + noise_j) where
 // noise holds the caller's Gumbel samples -- what jax.random.categorical evaluates.  One
 // workgroup per row: an 8-bit-per-pass radix select over order-preserving keys finds the k-th
 // largest key, elements above it are collected in any order, elements equal to it in index order.
@@ -1428,15 +1429,16 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
   }
   }
   }
-  // order the k candidates: value descending, index ascending
+  // order the k candidates: key descending (the order of the selection: -0 below +0), index ascending
   if (tid < p.k) {
     const float v = c_val[tid];
+    const uint32_t kv = topk_key(v);
     const int ix = c_idx[tid];
     int r = 0;
 #pragma unroll 16
     for (int j = 0; j < kTopKMax; ++j) {       // fixed trip count: the LDS reads go out in batches
-      const float vj = c_val[j];
-      r += (j < p.k && (vj > v || (vj == v && c_idx[j] < ix))) ? 1 : 0;
+      const uint32_t kj = topk_key(c_val[j]);
+      r += (j < p.k && (kj > kv || (kj == kv && c_idx[j] < ix))) ? 1 : 0;
     }
     o_val[r] = v;
     o_idx[r] = ix;

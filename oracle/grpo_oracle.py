@@ -36,6 +36,8 @@ Parity unpinned (documented, accepted):
   * JAX's half-gradient tie rule exactly at ratio == 1-eps_low / 1+eps_high
     (lax.min / lax.clip JVP); the closed form here takes the full unclipped
     gradient on the closed interval.
+  * How jax.lax.top_k orders -0 against +0 and where it puts NaNs: restated with the IEEE total
+    order of XLA's sort comparators (-0 < +0, NaN largest); only an import could confirm it.
   * Target ids outside [0, V): jnp.take_along_axis wraps negative ids and yields NaN
     past V; the oracle is only ever called with ids in range (the kernels clamp such
     ids, and their tests compare against the oracle on the clamped ids).
@@ -251,11 +253,15 @@ def top_k_sample(logits, k=50, t=0.9, noise=None):
     """_top_k_sampling_batched (MLLM_JAX/sample/sanple_utils.py:35-53) with the categorical draw
     written as argmax(top_logits + Gumbel noise) (what jax.random.categorical evaluates).
     logits [B,V] float32; scaled = logits / float32(t) in float32 (the reference divides, :37); top-k in descending order,
-    equal values by ascending index (jax.lax.top_k); noise [B,k] or None (greedy).
+    equal entries by ascending index (jax.lax.top_k); noise [B,k] or None (greedy).
     Returns (token[B], top_idx[B,k], top_val[B,k])."""
     x = np.asarray(logits, np.float32) / np.float32(t)
     b, v = x.shape
-    order = np.lexsort((np.broadcast_to(np.arange(v), x.shape), -x.astype(np.float64)), axis=-1)[:, :k]
+    # descending in the IEEE total order (-0 below +0, a NaN with the sign bit clear above +inf), the
+    # order XLA's sort comparators give floats; equal keys by ascending index
+    bits = x.view(np.uint32)
+    key = np.where(bits & np.uint32(0x80000000), ~bits, bits | np.uint32(0x80000000)).astype(np.int64)
+    order = np.lexsort((np.broadcast_to(np.arange(v), x.shape), -key), axis=-1)[:, :k]
     top_val = np.take_along_axis(x, order, axis=-1)
     if noise is None:
         pick = np.zeros(b, np.int64)

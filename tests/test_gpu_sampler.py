@@ -72,6 +72,27 @@ def test_neighbouring_floats_that_divide_to_the_same_quotient(t):
     np.testing.assert_array_equal(tok.cpu().numpy(), rt)
 
 
+def test_signed_zeros_and_nans_follow_the_total_order():
+    """Rows of +0 / -0 / tiny values (the k-th place falls among zeros of both signs) and rows with
+    NaN and infinities: selection and order are those of the IEEE total order, as in the oracle."""
+    import mllm_jax_amd as M
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(11)
+    for v, k in ((50, 34), (129, 64), (5000, 50), (70000, 50)):
+        x = rng.normal(0, 1e-3, size=(6, v)).astype(np.float32)
+        x[:, ::7] = 0.0
+        x[:, 3::11] = -0.0
+        x[3] = np.where(rng.random(v) < 0.5, 0.0, -0.0).astype(np.float32)      # nothing but zeros
+        x[4, rng.integers(0, v, size=5)] = np.nan
+        x[5, rng.integers(0, v, size=3)] = np.inf
+        x[5, rng.integers(0, v, size=3)] = -np.inf
+        tok, idx, val = M.top_k_sampling_batched(None, torch.tensor(x, device=dev), k=k, t=1.3, return_top_k=True)
+        rt, ri, rv = O.top_k_sample(x, k=k, t=1.3, noise=None)
+        np.testing.assert_array_equal(idx.cpu().numpy(), ri)
+        np.testing.assert_array_equal(val.cpu().numpy().view(np.uint32), rv.view(np.uint32))
+        np.testing.assert_array_equal(tok.cpu().numpy(), rt)
+
+
 def test_ties_duplicates_and_negative_values():
     import mllm_jax_amd as M
     dev = torch.device("cuda:0")

@@ -377,6 +377,15 @@ def test_top_k_sample_against_torch_topk_and_by_hand(rng):
     np.testing.assert_array_equal(idx, [[1, 2, 4, 5]])
     np.testing.assert_array_equal(val, [[3.0, 3.0, 3.0, 2.0]])
     assert tok[0] == 4
+    # signed zeros and NaN by hand, in the IEEE total order: -0 below +0, a NaN (sign bit clear) above +inf
+    w = np.array([[0.0, -0.0, 1.0, -0.0, 0.0, -1.0]], np.float32)
+    _, idx, val = O.top_k_sample(w, k=5, t=1.0, noise=None)
+    np.testing.assert_array_equal(idx, [[2, 0, 4, 1, 3]])
+    np.testing.assert_array_equal(np.signbit(val), [[False, False, False, True, True]])
+    w = np.array([[2.0, np.nan, np.inf, -np.inf, 3.0]], np.float32)
+    tok, idx, _ = O.top_k_sample(w, k=3, t=1.0, noise=None)
+    np.testing.assert_array_equal(idx, [[1, 2, 4]])
+    assert tok[0] == 1
     # Gumbel-max over the top k follows softmax(top_logits): frequencies of a 3-way draw
     z = np.array([[np.log(0.6), np.log(0.3), np.log(0.1), -50.0]], np.float32)
     u = rng.random((20000, 3)); g = -np.log(-np.log(u))
