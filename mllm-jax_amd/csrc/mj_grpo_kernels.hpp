@@ -1254,9 +1254,9 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) rank += w[j] > mine ? 1 : 0;
       }
-      if (rank < p.k) { c_val[rank] = topk_unkey((uint32_t)(mine >> 32)); c_idx[rank] = (int)~(uint32_t)mine; }
+      // the rank is the final position: (key descending, index ascending) is the order of the result
+      if (rank < p.k) { o_val[rank] = topk_unkey((uint32_t)(mine >> 32)); o_idx[rank] = (int)~(uint32_t)mine; }
     }
-    __syncthreads();
   } else {
   // ---- two reads of the row with a 12-bit histogram: finds the bin of the k-th largest
   // key; a second read sends larger keys straight to the result and the bin's keys to an LDS pool,
@@ -1429,8 +1429,8 @@ __global__ __launch_bounds__(1024) void k_topk_sample(TopKArgs p) {
   }
   }
   }
-  // order the k candidates: key descending (the order of the selection: -0 below +0), index ascending
-  if (tid < p.k) {
+  // histogram paths: order the k candidates, key descending (-0 below +0), index ascending
+  if (ranked > (uint32_t)kRankPool && tid < p.k) {
     const float v = c_val[tid];
     const uint32_t kv = topk_key(v);
     const int ix = c_idx[tid];
