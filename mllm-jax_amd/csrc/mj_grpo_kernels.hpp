@@ -196,6 +196,13 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
           for (int r = 0; r < 16; ++r) g.acc[mi][ni][r] = softcap_apply(g.acc[mi][ni][r], p.cap, inv_cap);
       }
     }
+    // An opaque use of the block's 64 accumulators: with it the register allocator moves them out of
+    // the accumulation registers here, one block at a time, instead of parking 32 of them in scratch
+    // memory at the start of the epilogue (no scratch access is left in the kernel; measured 1 % faster).
+#pragma unroll
+    for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) asm volatile("" : "+v"(g.acc[mi][ni][r]));
     // The stand-in for rows past V is a rare, wave-uniform case behind a real scalar branch (the
     // empty asm keeps the compiler from flattening it into per-element selects).
     if (tail) {
