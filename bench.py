@@ -25,9 +25,9 @@ PEAK_HBM_GBS = 8000.0
 # a plain 1 GiB device copy (x2.00 fetch, x1.00 write); summary in profiles/.  Keyed by
 # (config index, kernel); None for workloads that were not counted.
 MEASURED_TRAFFIC_BYTES = {          # default chunk (16384 tokens: one launch of each kernel per step)
-    (2, "k_logits_stats"): 32.70e9,
-    (2, "k_dhidden"): 33.88e9,
-    (2, "k_dw"): 36.58e9,
+    (2, "k_logits_stats"): 31.38e9,
+    (2, "k_dhidden"): 34.44e9,
+    (2, "k_dw"): 37.51e9,
 }
 
 
