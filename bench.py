@@ -210,6 +210,30 @@ def _neighbours(torch, M, _lib, cfg, wl, dev, iters=20) -> dict:
         torch.matmul(last, w)
         return 0
     calls["vendor_matmul_for_sample_logits"] = (vendor_product, h * v * 2 + b_seq * h * 2 + b_seq * v * 2)
+    # what plain streaming reaches on this GPU beyond the 256 MB Infinity Cache: the value head (read
+    # only) and the RMSNorm forward (read + write) on a 1.07 GB matrix, and torch's own sum and copy
+    # over 1 GiB -- yardsticks for the fractions of the nominal 8 TB/s above
+    bn_, bh_ = 131072, 4096
+    bigx = torch.empty((bn_, bh_), dtype=torch.bfloat16, device=dev).normal_()
+    bigy = torch.empty_like(bigx)
+    bigw, bigs, bigv = torch.full((bh_,), 0.01, **f32), torch.ones(bh_, **f32), torch.empty(bn_, **f32)
+    calls["stream_read_1GB_value_head_yardstick"] = (
+        lambda: lib.mj_value_head_forward(bigx.data_ptr(), bh_, bigw.data_ptr(), bv.data_ptr(), bigv.data_ptr(), bn_, bh_, st),
+        bn_ * bh_ * 2)
+    calls["stream_read_write_1GB_rmsnorm_yardstick"] = (
+        lambda: lib.mj_rmsnorm_forward(bigx.data_ptr(), bh_, bigs.data_ptr(), bigy.data_ptr(), bh_, None, bn_, bh_, 1e-6, st),
+        2 * bn_ * bh_ * 2)
+    bigf = bigx.view(torch.float32)
+
+    def torch_read():
+        torch.sum(bigf)
+        return 0
+
+    def torch_copy():
+        bigy.copy_(bigx)
+        return 0
+    calls["torch_sum_1GB_read_yardstick"] = (torch_read, bn_ * bh_ * 2)
+    calls["torch_copy_1GB_read_plus_write_yardstick"] = (torch_copy, 2 * bn_ * bh_ * 2)
     rows = {}
     for name, (fn, nbytes) in calls.items():
         for _ in range(3):
