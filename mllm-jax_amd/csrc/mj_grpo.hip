@@ -242,7 +242,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
   // Which statistics the logits epilogue keeps (mj::StatsMode): sums of exp(z) without a running
   // maximum plus E = exp(z) for the backward -- with a kStatsMax rescue pass enqueued behind it that
   // leaves at once unless the range check failed -- or, where that form does not apply, kStatsMax.
-  const bool exp_mode = mode != kBackwardOnly && d->temperature == 1.0f && d->entropy_coef == 0.f;
+  const bool exp_mode = mode != kBackwardOnly && d->entropy_coef == 0.f;
   int* state = (int*)(ws + p.state);
   float* rs = (float*)(ws + p.rs);
   uint16_t* hs = (uint16_t*)(ws + p.hs);

@@ -84,8 +84,8 @@ MJ_DEV int live_pad(const int* n_live, int c0, int n_pad) {
 //                backward products read E as it is: k_dhidden scales its output rows by rs_t, k_dw
 //                reads rs_t * hidden, and no pass over [n, V] is needed to form dZ.
 //   kStatsMax  : the same sums relative to the per-tile maximum (any logit range) and the capped
-//                logits as IEEE half; k_dz turns those into dZ in place.  Used with temperature != 1,
-//                with the entropy bonus, and as the rescue when kStatsExp's range check fails.
+//                logits as IEEE half; k_dz turns those into dZ in place.  Used with the entropy
+//                bonus and as the rescue when kStatsExp's range check fails.
 //   kStatsGrad : backward from a saved forward: lse and dloss/dlogp are inputs, so the epilogue writes
 //                dZ = -g * p * cap' directly (k_patch_grad adds the one-hot term).
 // state[0] tells the backward products what the 16-bit matrix holds: 0 = E (scale by rs, read
@@ -103,7 +103,7 @@ struct LogitsArgs {
   uint16_t* zt;          // [n, ld_z] 16-bit rows of the chunk (see StatsMode), or nullptr (forward only)
   int64_t ld_z;
   float *pm, *pl, *ps;   // per (vocab half-tile, token) partial max / sum e / sum e*z, ld = ld_p
-  float* plt;            // temperature != 1 only: sum e^((z-max)/T), and ps then holds sum e^((z-max)/T)*z
+  float* plt;            // temperature != 1 only: sum e^((z-max)/T), and ps then holds sum e^((z-max)/T)*z (max = 0 in kStatsExp)
   float inv_t;           // 1 / temperature
   int64_t ld_p;
   const int32_t* targets;   // chunk origin
@@ -307,12 +307,31 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
             s = fmaf(e, z, s);
           }
       }
+      float lt = 0.f;
+      if (p.inv_t != 1.f) {
+        // the entropy is that of softmax(z / T) (train_modules/__init__.py:136): its own pair of sums,
+        // behind a real scalar branch so that the usual T = 1 pays nothing for it
+        asm volatile("");
+        const float kt = kLog2e * p.inv_t;
+        s = 0.f;
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float z = g.acc[mi][ni][r];
+            const float e = __builtin_amdgcn_exp2f(z * kt);
+            lt += e;
+            s = fmaf(e, z, s);
+          }
+        lt += __shfl_xor(lt, 32);
+      }
       l += __shfl_xor(l, 32);
       s += __shfl_xor(s, 32);
       if (lhi == 0) {
         const int64_t o = (int64_t)(tm * 2 + wm) * p.ld_p + col;
         p.pl[o] = l;
         p.ps[o] = s;
+        if (p.inv_t != 1.f) p.plt[o] = lt;
       }
     } else {   // kStatsGrad
       const float lse2 = col < p.n ? p.lse[col] * kLog2e : 0.f;
@@ -423,6 +442,7 @@ __global__ __launch_bounds__(kFinTokens * kFinSlices) void k_finalize(FinalizeAr
       if (MODE == kStatsExp) {
         l += p.pl[o];
         s += p.ps[o];
+        if (tempered) lt += p.plt[o];
       } else {
         const float mq = p.pm[o], lq = p.pl[o], sq = p.ps[o];
         const float mn = fmaxf(m, mq);
@@ -454,9 +474,11 @@ __global__ __launch_bounds__(kFinTokens * kFinSlices) void k_finalize(FinalizeAr
     for (int i = 0; i < kFinSlices; ++i) {
       L += sl[i][tx];
       S += ss[i][tx];
+      LT += st[i][tx];
     }
     // outside the window (or not finite): the sums cannot be trusted; the kStatsMax pass redoes the chunk
     if (!(L >= kExpSumMin && L <= kExpSumMax)) *p.state = 1;
+    if (tempered && !(LT >= kExpSumMin && LT <= kExpSumMax)) *p.state = 1;
   } else {
     M = sm[0][tx];
 #pragma unroll

@@ -222,6 +222,24 @@ def test_logits_outside_the_exp_window_take_the_rescue_pass(shift):
     np.testing.assert_array_equal(fwd["token_entropy"].cpu().numpy().reshape(-1), met["token_entropy"].reshape(-1))
 
 
+@pytest.mark.parametrize("shift,temperature", [(30.0, 0.3), (-30.0, 0.3), (40.0, 2.0)])
+def test_tempered_sums_have_their_own_range_check(shift, temperature):
+    """T != 1: the entropy's sums run over exp(z / T).  With T = 0.3 a logit offset of +-30 keeps
+    sum exp(z) inside the window while exp(z / T) = exp(+-100) overflows or vanishes in float32, so the
+    second check must send the chunk to the running-maximum pass; with T = 2 and +40 both sums stay
+    inside.  Either way: the oracle."""
+    n, h, v, b = 512, 64, 1000, 2
+    hid, w, y, adv, mask = _case(23, n, h, v, b)
+    w = w.float()
+    w[0, :] = 1.0
+    hid = hid.float()
+    hid[:, 0] = 0.0
+    hid[256:, 0] = shift
+    hid, w = hid.to(torch.bfloat16), w.to(torch.bfloat16)
+    old = _old_from(_ref_logp(hid, w, y, temperature=temperature), 24)
+    _check(hid, w, y, old, adv, mask, seq_shape=(b, n // b), chunk_tokens=256, temperature=temperature)
+
+
 def test_deterministic_and_accumulate():
     import mllm_jax_amd as M
     d = _dev()
