@@ -276,6 +276,9 @@ def main() -> int:
                          "kernels + the in-place dZ pass instead of the default path")
     ap.add_argument("--dw-dtype", choices=("f32", "bf16"), default="f32",
                     help="dtype of the lm_head gradient the dW kernel writes (the reference's is float32: the default)")
+    ap.add_argument("--graph", action="store_true",
+                    help="capture one step in a HIP graph and time its replays (small shapes are launch-bound; implies "
+                         "--no-kernel-events: the per-kernel timers then run in a separate eager loop)")
     ap.add_argument("--neighbours", action="store_true",
                     help="instead of the loss step, time the steps either side of it (RMSNorm, sampler, value head, "
                          "group advantages) at the config's shape against the HBM roofline")
@@ -356,6 +359,28 @@ def main() -> int:
     torch.cuda.synchronize()
     if 64 * args.steps > 60000:          # more event pairs than the library's profiler takes (65536)
         args.no_kernel_events = True
+    eager_step = step
+    if args.graph:
+        # the library's calls record into a capturing stream as they are (no allocation, no host
+        # synchronisation; the first calls above ran outside the capture)
+        args.no_kernel_events = True
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                eager_step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            captured = eager_step()
+
+        def step():
+            graph.replay()
+            return captured
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
     if not args.no_kernel_events:
         _lib.profile_begin(64 * max(args.steps, 1))
     sampler = _SmiSampler() if args.smi else None
@@ -376,7 +401,7 @@ def main() -> int:
         prof_steps = min(args.steps, 5)
         _lib.profile_begin(64 * prof_steps)
         for _ in range(prof_steps):
-            step()
+            eager_step()
         torch.cuda.synchronize()
     prof = _lib.profile_end()
 
@@ -424,16 +449,18 @@ def main() -> int:
         line["config"]["kernel_events"] = "separate loop of %d steps after the timed one" % prof_steps
     if args.entropy_coef:
         line["config"]["entropy_coef"] = args.entropy_coef
+    if args.graph:
+        line["config"]["launch"] = "replays of one HIP graph of the step"
     line["config"]["skip_masked"] = bool(args.skip_masked)
     if not args.skip_masked and not args.no_skip_masked_extra:
         # Not the headline: the same step with tokens that cannot carry a gradient (mask 0, advantage 0)
         # left out of the backward products.  Same outputs; fewer than 6*N*H*V flop executed.
         for _ in range(2):
-            step(True)
+            eager_step(True)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         for _ in range(5):
-            step(True)
+            eager_step(True)
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t1) / 5 * 1e3
         live = float(((wl["mask"] != 0) & (wl["advantages"].reshape(wl["mask"].shape) != 0)).float().mean().item())
