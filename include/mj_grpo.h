@@ -50,7 +50,8 @@ enum {
                                            -logp, advantages/old_logp ignored */
   MJ_GRPO_FLAG_SKIP_MASKED = 1u << 2,   /* tokens whose gradient is zero by construction (mask 0: prompt
                                            and padding positions, labels of train_modules/__init__.py:120;
-                                           advantage 0 when nothing else feeds the gradient) are moved
+                                           advantage 0 when nothing else feeds the gradient, i.e. no entropy
+                                           bonus and no value head) are moved
                                            behind the others and left out of the backward products.
                                            Same outputs (d_lm_head up to summation order); the forward
                                            still covers every token.  No counterpart in the reference,

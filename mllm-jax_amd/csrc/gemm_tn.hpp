@@ -115,7 +115,10 @@ struct TileMap {
 
 // One operand of the tile: ROWS tile rows (M or N direction) by 64 k per slice, 128*ROWS bytes of
 // LDS per stage, ROWS*8/THREADS 16-byte chunks per thread per slice.
-template <int ROWS, int LAYOUT, int THREADS>
+// DEAD: the caller knows which rows (kRowK) or k-rows (kKRow) of the operand are all zero and hands
+// in a bit mask, one 64-bit word per 64 of them (bit set = zero, do not fetch).  Their loads get an
+// offset that the descriptor rejects: the registers fill with zeros and no memory request is made.
+template <int ROWS, int LAYOUT, int THREADS, bool DEAD = false>
 struct Operand {
   static constexpr int LD = ROWS * 8 / THREADS;
   static constexpr int RPP = THREADS / 8;          // kRowK: tile rows covered by one pass of the workgroup
@@ -139,9 +142,13 @@ struct Operand {
   // 16-byte chunk permutation of the kRowK image (see the file header).
   static MJ_DEV int swz(int r) { return (r & 7) ^ ((r >> 3) & 3); }   // depends on r mod 32 only
 
-  MJ_DEV void init(const __bf16* p, int rows_valid, int64_t ld, int K_, int wave_row0) {
+  // dead: kRowK -- the words covering this tile's ROWS rows (ROWS / 64 of them);
+  //       kKRow -- the words of the K extent, one per slice ((K + 63) / 64 of them).
+  MJ_DEV void init(const __bf16* p, int rows_valid, int64_t ld, int K_, int wave_row0, int t,
+                   const uint64_t* dead = nullptr) {
     static_assert(LAYOUT == kRowK || ROWS == 256, "the k-major image is laid out for 256-row tiles");
-    const int t = threadIdx.x, lane = t & 63;
+    static_assert(!DEAD || (ROWS == 256 && THREADS == 256), "the dead-row masks assume 8 chunks per thread, 32 or 8 rows apart");
+    const int lane = t & 63;
     base = (const char*)p;
     ld2 = ld * 2;
     rows = rows_valid < ROWS ? rows_valid : ROWS;
@@ -151,6 +158,12 @@ struct Operand {
       rsrc = make_rsrc(base, (int64_t)rows * ld2);
 #pragma unroll
       for (int i = 0; i < LD; ++i) goff[i] = (uint32_t)((row + RPP * i) * ld2 + chunk * 16);
+      if (DEAD) {
+        // rows row + 32 i: bit row + 32 (i & 1) of word i / 2
+#pragma unroll
+        for (int i = 0; i < LD; ++i)
+          if ((dead[i >> 1] >> (row + 32 * (i & 1))) & 1ull) goff[i] = kOob;
+      }
       klimit = K - chunk * 8;
       st_off = row * 128 + ((chunk ^ swz(row)) << 4);   // swz(row + RPP*i) == swz(row)
       st_off1 = st_off;
@@ -189,12 +202,16 @@ struct Operand {
       rsrc = make_rsrc(base + (int64_t)k0 * ld2, (int64_t)(left < kBK ? left : kBK) * ld2);
     }
   }
-  MJ_DEV u32x4 load(int slice, int i) const {
+  // dead_lo / dead_hi (DEAD && kKRow): KDead's bits for the slice
+  MJ_DEV u32x4 load(int slice, int i, uint32_t dead_lo = 0, uint32_t dead_hi = 0) const {
     if (LAYOUT == kRowK) {
       const int k0 = slice * kBK;
       return __builtin_amdgcn_raw_buffer_load_b128(rsrc, k0 < klimit ? goff[i] : kOob, k0 * 2, 0);
     }
-    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, col_ok ? goff[i] : kOob, 0, 0);
+    uint32_t off = col_ok ? goff[i] : kOob;
+    if (DEAD)   // bit 8 (i % 4) of the shifted word set: the offset becomes one that every descriptor rejects
+      off |= (uint32_t)__builtin_amdgcn_sbfe((int)(i < 4 ? dead_lo : dead_hi), 8 * (i & 3), 1) & kOob;
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
   }
   MJ_DEV void store(char* stage, int i, u32x4 v) const {
     if (LAYOUT == kRowK)
@@ -217,19 +234,49 @@ struct Operand {
 template <int V>
 struct IntTag { static constexpr int value = V; };
 
+// Mask of all-zero k-rows for operands in the kKRow layout (256-row tiles, 256 threads: a thread
+// loads chunk i of a slice from k-row t / 32 + 8 i).  One 64-bit word per slice, bit r set = k-row r
+// of the slice is zero.  The word of the next slice is requested while the current one is used;
+// lo / hi hold the current word shifted so that bit 8 (i % 4) of (i < 4 ? lo : hi) is chunk i's row.
+struct KDead {
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint64_t next;
+  uint32_t lo, hi;
+  int krow;
+  MJ_DEV uint64_t word(int slice) const {
+    typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+    const u32x2 w = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rsrc, 0, slice * 8, 0));
+    return ((uint64_t)w[1] << 32) | w[0];
+  }
+  MJ_DEV void init(const uint64_t* words, int K, int t) {
+    krow = t >> 5;
+    rsrc = make_rsrc(words, (int64_t)((K + kBK - 1) / kBK) * 8);   // words past K read 0: nothing to skip
+    next = word(0);
+    lo = hi = 0;
+  }
+  MJ_DEV void slice_begin(int slice) {
+    const uint64_t w = next >> krow;
+    lo = (uint32_t)w;
+    hi = (uint32_t)(w >> 32);
+    next = word(slice + 1);
+  }
+};
+
 // DEPTH: slices in flight between global memory and the LDS.  1: the loads of slice k+2 are issued
 // during slice k and written to the LDS during slice k+1 (one slice of math to land).  2: a second
 // set of staging registers; the loads of slice k+3 are issued during slice k and written during
 // slice k+2 (two slices to land) -- for shapes whose operands come from HBM on every slice.
-template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK, int DEPTH = 1, int WAVES_M = 2, int WAVES_N = 2>
+// DEAD_A / DEAD_B: the operand takes a mask of rows (kRowK) or k-rows (kKRow) known to be zero.
+template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK, int DEPTH = 1, bool DEAD_A = false,
+          bool DEAD_B = false, int WAVES_M = 2, int WAVES_N = 2>
 struct GemmTN {
   static_assert(BM % 32 == 0 && BN % 32 == 0, "tile sides are multiples of 32");
   static constexpr int kWavesM = WAVES_M, kWavesN = WAVES_N;
   static constexpr int kThreads = 64 * WAVES_M * WAVES_N;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;   // wavefront tile
   static constexpr int MI = WM / 32, NI = WN / 32;   // 32x32 blocks per wavefront
-  using OpA = Operand<BM, LAY_A, kThreads>;
-  using OpB = Operand<BN, LAY_B, kThreads>;
+  using OpA = Operand<BM, LAY_A, kThreads, DEAD_A>;
+  using OpB = Operand<BN, LAY_B, kThreads, DEAD_B>;
   static constexpr int A_LD = OpA::LD, B_LD = OpB::LD;
   static constexpr int LPS = A_LD + B_LD;            // 16-byte chunks per thread per slice
   static constexpr int kStageBytes = OpA::kBytes + OpB::kBytes;
@@ -242,23 +289,40 @@ struct GemmTN {
 
   // A, B: tile origin pointers (row 0 of the tile, k = k_begin); rows_*: valid rows of the tile;
   // ld*: elements between rows (kRowK) or between k-rows (kKRow); K: k extent from the origin.
+  // tid: the thread's index in the workgroup (a kernel that loops over tiles passes a value the
+  // compiler cannot see through, so that the per-thread address arithmetic is redone per tile
+  // instead of living in registers across the epilogue).
+  static constexpr bool kKDead = (DEAD_A && LAY_A == kKRow) || (DEAD_B && LAY_B == kKRow);
+  static_assert(!kKDead || (BM == 256 && BN == 256 && LAY_A == kKRow && LAY_B == kKRow && DEAD_A && DEAD_B),
+                "a k-row mask covers both operands of a 256 x 256 tile");
+
+  // dead_a / dead_b: see Operand::init and KDead (only read when DEAD_A / DEAD_B; a k-row mask is
+  // one list, passed as dead_a).
   MJ_DEV void run(const __bf16* A, int rows_a, int64_t lda, const __bf16* B, int rows_b,
-                  int64_t ldb, int K, char* smem) {
+                  int64_t ldb, int K, char* smem, int tid = threadIdx.x, const uint64_t* dead_a = nullptr,
+                  const uint64_t* dead_b = nullptr) {
     if (DEPTH == 2) {
-      run_deep(A, rows_a, lda, B, rows_b, ldb, K, smem);
+      run_deep(A, rows_a, lda, B, rows_b, ldb, K, smem, tid, dead_a, dead_b);
       return;
     }
-    const int wave = threadIdx.x >> 6;
+    const int wave = tid >> 6;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     OpA a;
     OpB b;
-    a.init(A, rows_a, lda, K, wm * WM);
-    b.init(B, rows_b, ldb, K, wn * WN);
+    a.init(A, rows_a, lda, K, wm * WM, tid, dead_a);
+    b.init(B, rows_b, ldb, K, wn * WN, tid, dead_b);
+    KDead kd;
+    if (kKDead) kd.init(dead_a, K, tid);
+    auto slices_begin = [&](int slice) {
+      a.slice_begin(slice);
+      b.slice_begin(slice);
+      if (kKDead) kd.slice_begin(slice);
+    };
 
     u32x4 staged[LPS];
     auto load_one = [&](int slice, int j) {
-      if (j < A_LD) staged[j] = a.load(slice, j);
-      else staged[j] = b.load(slice, j - A_LD);
+      if (j < A_LD) staged[j] = kKDead ? a.load(slice, j, kd.lo, kd.hi) : a.load(slice, j);
+      else staged[j] = kKDead ? b.load(slice, j - A_LD, kd.lo, kd.hi) : b.load(slice, j - A_LD);
     };
     auto store_one = [&](int slice, int j) {
       char* stage = smem + (slice & 1) * kStageBytes;
@@ -302,12 +366,10 @@ struct GemmTN {
 
     static_assert(LPS <= 3 * G, "the staged chunks of a slice must fit the first three k-steps");
     const int KT = (K + kBK - 1) / kBK;
-    a.slice_begin(0);
-    b.slice_begin(0);
+    slices_begin(0);
 #pragma unroll
     for (int j = 0; j < LPS; ++j) load_one(0, j);
-    a.slice_begin(1);
-    b.slice_begin(1);
+    slices_begin(1);
 #pragma unroll
     for (int j = 0; j < LPS; ++j) {
       store_one(0, j);
@@ -319,8 +381,7 @@ struct GemmTN {
     for (int g = 0; g < G; ++g) read_one(0, 0, 0, g);
     for (int kt = 0; kt < KT; ++kt) {
       // slice kt+1 moves registers -> the stage slice kt-1 occupied; slice kt+2 starts loading
-      a.slice_begin(kt + 2);
-      b.slice_begin(kt + 2);
+      slices_begin(kt + 2);
       kstep(0, kt, 1, kt, 0);
       kstep(1, kt, 2, kt, G);
       kstep(0, kt, 3, kt, 2 * G);
@@ -335,19 +396,26 @@ struct GemmTN {
   // (kt+1) & 1 and refills that set with slice kt+3; the loop is unrolled by two so that the set
   // index is a compile-time constant.
   MJ_DEV void run_deep(const __bf16* A, int rows_a, int64_t lda, const __bf16* B, int rows_b, int64_t ldb,
-                       int K, char* smem) {
-    const int wave = threadIdx.x >> 6;
+                       int K, char* smem, int tid, const uint64_t* dead_a, const uint64_t* dead_b) {
+    const int wave = tid >> 6;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     OpA a;
     OpB b;
-    a.init(A, rows_a, lda, K, wm * WM);
-    b.init(B, rows_b, ldb, K, wn * WN);
+    a.init(A, rows_a, lda, K, wm * WM, tid, dead_a);
+    b.init(B, rows_b, ldb, K, wn * WN, tid, dead_b);
+    KDead kd;
+    if (kKDead) kd.init(dead_a, K, tid);
+    auto slices_begin = [&](int slice) {
+      a.slice_begin(slice);
+      b.slice_begin(slice);
+      if (kKDead) kd.slice_begin(slice);
+    };
 
     u32x4 staged[2][LPS];
     auto load_one = [&](auto set, int slice, int j) {
       constexpr int S = decltype(set)::value;
-      if (j < A_LD) staged[S][j] = a.load(slice, j);
-      else staged[S][j] = b.load(slice, j - A_LD);
+      if (j < A_LD) staged[S][j] = kKDead ? a.load(slice, j, kd.lo, kd.hi) : a.load(slice, j);
+      else staged[S][j] = kKDead ? b.load(slice, j - A_LD, kd.lo, kd.hi) : b.load(slice, j - A_LD);
     };
     auto store_one = [&](auto set, int slice, int j) {
       constexpr int S = decltype(set)::value;
@@ -378,8 +446,7 @@ struct GemmTN {
       }
     };
     auto iteration = [&](auto set, int kt) {
-      a.slice_begin(kt + 3);
-      b.slice_begin(kt + 3);
+      slices_begin(kt + 3);
       kstep(set, 0, kt, 1, kt, 0);
       kstep(set, 1, kt, 2, kt, G);
       kstep(set, 0, kt, 3, kt, 2 * G);
@@ -397,16 +464,13 @@ struct GemmTN {
         for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
 
     const int KT = (K + kBK - 1) / kBK;
-    a.slice_begin(0);
-    b.slice_begin(0);
+    slices_begin(0);
 #pragma unroll
     for (int j = 0; j < LPS; ++j) load_one(IntTag<0>(), 0, j);
-    a.slice_begin(1);
-    b.slice_begin(1);
+    slices_begin(1);
 #pragma unroll
     for (int j = 0; j < LPS; ++j) load_one(IntTag<1>(), 1, j);
-    a.slice_begin(2);
-    b.slice_begin(2);
+    slices_begin(2);
 #pragma unroll
     for (int j = 0; j < LPS; ++j) {
       store_one(IntTag<0>(), 0, j);

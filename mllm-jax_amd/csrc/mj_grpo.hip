@@ -64,7 +64,7 @@ struct Plan {
   int dh_splits;          // vocab splits of the dHidden product (1 = none)
   int64_t dh_k_per_split;
   // byte offsets into the workspace
-  size_t zy, term, eterm, pm, pl, ps, plt, g, ge, hent, state, rs, hs, zt, part, total_fwd, total_bwd;
+  size_t zy, term, eterm, pm, pl, ps, plt, g, ge, hent, state, rs, dead, hs, zt, part, total_fwd, total_bwd;
   // token compaction (MJ_GRPO_FLAG_SKIP_MASKED): slot-order copies of the inputs and outputs
   bool compact;
   size_t perm, n_live, hid_p, tgt_p, fin_p[5], fout_p[3], dh_p;
@@ -146,6 +146,7 @@ int make_plan(const MjGrpoDesc* d, Plan* p) {
   p->total_fwd = o;
   p->dh_p = take(p->compact ? (size_t)p->N * p->H * 2 : 0);
   p->rs = take((size_t)p->n_pad * 4);
+  p->dead = take((size_t)p->n_pad / 8);     // one bit per token of a chunk
   p->hs = take((size_t)p->n_pad * p->H * 2);
   p->zt = take((size_t)p->n_pad * p->ld_z * 2);
   p->part = take(p->dh_splits > 1 ? (size_t)p->dh_splits * p->n_pad * p->H * 4 : 0);
@@ -246,6 +247,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
   int* state = (int*)(ws + p.state);
   float* rs = (float*)(ws + p.rs);
   uint16_t* hs = (uint16_t*)(ws + p.hs);
+  uint64_t* dead = (uint64_t*)(ws + p.dead);
   // the logits kernels exist with and without the softcap code (a template parameter)
   const bool cap = d->softcap > 0.f;
   auto k_grad = cap ? mj::k_logits_stats<BM, BN, mj::kStatsGrad, false, true> : mj::k_logits_stats<BM, BN, mj::kStatsGrad, false, false>;
@@ -298,7 +300,9 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     perm = (const int*)(ws + p.perm);
     n_live = (const int*)(ws + p.n_live);
     mj::CompactArgs c;
-    c.mask = mask; c.adv = (sft || d->entropy_coef != 0.f) ? nullptr : adv; c.n = N;
+    // a token with advantage exactly 0 is dead only when nothing else feeds its gradient: the entropy
+    // bonus and the critic's dv[t] * value_w both reach d_hidden[t, :] whatever the advantage is
+    c.mask = mask; c.adv = (sft || d->entropy_coef != 0.f || pv != nullptr) ? nullptr : adv; c.n = N;
     c.perm = (int*)(ws + p.perm); c.n_live = (int*)(ws + p.n_live);
     mj::k_compact_plan<<<1, 1024, 0, st>>>(c);
     mj::GatherArgs ga;
@@ -348,12 +352,12 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
     f.ent_coef = d->entropy_coef; f.inv_ent_cnt = d->inv_entropy_count; f.eterm = eterm + c0;
     f.ge = bonus ? ge : nullptr; f.hent = bonus ? hent : nullptr;
     f.rs = bwd ? rs : nullptr; f.zt = zt; f.ld_z = p.ld_z; f.targets = targets + c0; f.V = V; f.cap = d->softcap;
-    f.state = state; f.rescue = 0;
+    f.state = state; f.rescue = 0; f.dead = bwd ? (uint16_t*)dead : nullptr;
 
     mj::DzArgs z;
     z.zt = zt; z.ld_z = p.ld_z;
     z.lse = (mode == kBackwardOnly ? saved_lse : lse) + c0; z.g = g; z.targets = targets + c0;
-    z.ge = bonus ? ge : nullptr; z.hent = bonus ? hent : nullptr;
+    z.ge = bonus ? ge : nullptr; z.hent = bonus ? hent : nullptr; z.mask = mask + c0;
     z.V = V; z.n = nc; z.cap = d->softcap; z.n_live = n_live; z.c0 = (int)c0; z.state = state; z.rescue = 0;
     const unsigned dz_grid = (unsigned)(nc < 8192 ? nc : 8192);
 
@@ -362,7 +366,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
         Timed t(MJ_GRPO_K_FINALIZE, st);
         mj::k_coeff_from_saved<<<(n_pad + 255) / 256, 256, 0, st>>>(
             saved_logp + c0, old_logp ? old_logp + c0 : nullptr, adv ? adv + c0 : nullptr, mask + c0, nc, n_pad,
-            d->eps_low, d->eps_high, d->inv_total_valid_tokens, gscale * inv_t, sft ? 1 : 0, g);
+            d->eps_low, d->eps_high, d->inv_total_valid_tokens, gscale * inv_t, sft ? 1 : 0, g, dead);
       }
       a.lse = saved_lse + c0;
       {
@@ -416,7 +420,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       h.splits = p.dh_splits; h.k_per_split = (int)p.dh_k_per_split;
       h.dh = (uint16_t*)d_hidden + c0 * ld_dh; h.ld_dh = ld_dh;
       h.part = part; h.n_live = n_live; h.c0 = (int)c0; h.rs = rs; h.state = state;
-      h.dv = dv ? dv + c0 : nullptr; h.wv = pv ? pv->value_w : nullptr;
+      h.dv = dv ? dv + c0 : nullptr; h.wv = pv ? pv->value_w : nullptr; h.dead = dead;
       const mj::TileMap mh = mj::TileMap::pick_shape((nc + BM - 1) / BM, (H + BN - 1) / BN, 0, h.splits);
       {
         Timed t(MJ_GRPO_K_DHIDDEN, st);
@@ -432,7 +436,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
       mj::DwArgs w;
       w.dzt = (const __bf16*)zt; w.hid = hid_c; w.hs = (const __bf16*)hs; w.ld_z = p.ld_z; w.ld_hid = ld_hid;
       w.H = H; w.V = V; w.n = nc;
-      w.dw = d_w; w.ld_dw = d->ld_w; w.n_live = n_live; w.c0 = (int)c0; w.state = state;
+      w.dw = d_w; w.ld_dw = d->ld_w; w.n_live = n_live; w.c0 = (int)c0; w.state = state; w.dead = dead;
       w.accumulate = (c0 > 0 || (d->flags & MJ_GRPO_FLAG_DW_ACCUMULATE)) ? 1 : 0;
       const mj::TileMap mw = mj::TileMap::pick_shape((V + BM - 1) / BM, (H + BN - 1) / BN, 0, 1);
       {

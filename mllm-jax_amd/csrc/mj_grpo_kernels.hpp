@@ -79,7 +79,7 @@ MJ_DEV int live_pad(const int* n_live, int c0, int n_pad) {
 //   kStatsExp  : per (vocab half-tile, token) the sums of e = exp(z) and e * z with NO running
 //                maximum (valid while logsumexp(z) stays within +-60, which k_finalize checks for
 //                every token) and, when a backward follows, the row-major 16-bit matrix
-//                E[t, v] = bf16(exp(z) * cap'(z)) with zero rows for masked tokens.  Since
+//                E[t, v] = bf16(exp(z) * cap'(z)); rows of masked tokens are not written.  Since
 //                dZ[t, v] = rs_t * (E[t, v] - onehot patch) with rs_t = -g_t / sum_v exp(z), the two
 //                backward products read E as it is: k_dhidden scales its output rows by rs_t, k_dw
 //                reads rs_t * hidden, and no pass over [n, V] is needed to form dZ.
@@ -89,7 +89,10 @@ MJ_DEV int live_pad(const int* n_live, int c0, int n_pad) {
 //   kStatsGrad : backward from a saved forward: lse and dloss/dlogp are inputs, so the epilogue writes
 //                dZ = -g * p * cap' directly (k_patch_grad adds the one-hot term).
 // state[0] tells the backward products what the 16-bit matrix holds: 0 = E (scale by rs, read
-// rs * hidden), 1 = dZ itself.
+// rs * hidden), 1 = dZ itself.  Either way the rows of tokens without a gradient (dloss/dlogp and
+// the entropy-bonus coefficient both 0: masked tokens, zero advantages) are never read: one bit
+// per token, 64-bit words (`dead`), tells the loaders of the backward products to fill those rows
+// with zeros instead of fetching them.  The products still multiply the zeros.
 enum StatsMode { kStatsExp = 0, kStatsMax = 1, kStatsGrad = 2 };
 
 constexpr float kExpSumMin = 0x1p-86f, kExpSumMax = 0x1p86f;   // logsumexp within about +-59.6
@@ -110,7 +113,7 @@ struct LogitsArgs {
   float* zy;                // chunk origin: capped logit of the sampled token
   const int* n_live;        // null, or device count of leading tokens (from token c0 on) that need a backward
   int c0;
-  const float* mask;        // kStatsExp: chunk origin; tokens with mask == 0 get zero rows of E
+  const float* mask;        // chunk origin; rows of tokens with mask == 0 are not stored
   const float *lse, *g;     // kStatsGrad: chunk-local saved logsumexp [n] and dloss/dlogp [n_pad]
   int* state;
 };
@@ -132,7 +135,7 @@ MJ_DEV uint32_t pack_f16(float a, float b) {   // clamped to the finite half ran
 // one half with the partner each lane owns eight CONSECUTIVE vocab entries and stores them with
 // one 16-byte access (`voff` carries the lane's 16 bytes of the 32).
 template <bool HALF>
-MJ_DEV void store_rows8(const float (&v)[8], uint32_t keep, __amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff) {
+MJ_DEV void store_rows8(const float (&v)[8], __amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff) {
   uint32_t a0, a1, b0, b1;
   if (HALF) {
     a0 = pack_f16(v[0], v[1]); a1 = pack_f16(v[2], v[3]); b0 = pack_f16(v[4], v[5]); b1 = pack_f16(v[6], v[7]);
@@ -142,20 +145,20 @@ MJ_DEV void store_rows8(const float (&v)[8], uint32_t keep, __amdgpu_buffer_rsrc
   // v_permlane32_swap: the first operand of lanes 32..63 <-> the second operand of lanes 0..31
   const auto s0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
   const auto s1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
-  const u32x4 out = {s0[0] & keep, s1[0] & keep, s0[1] & keep, s1[1] & keep};
+  const u32x4 out = {s0[0], s1[0], s0[1], s1[1]};
   __builtin_amdgcn_raw_buffer_store_b128(out, rs, voff, soff, 0);
 }
 
 // One 256 x 256 tile: logits^T [vocab x tokens] = W^T * hidden^T on MFMA, then the epilogue of MODE.
 template <int BM, int BN, int MODE, bool CAP>
-MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
+MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid) {
   using G = GemmTN<BM, BN, kKRow, kRowK>;
   const int m0 = tm * BM, n0 = tn * BN;
   G g;
-  g.run(p.w + m0, p.V - m0, p.ld_w, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0, p.ld_hid, p.H, smem);
+  g.run(p.w + m0, p.V - m0, p.ld_w, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0, p.ld_hid, p.H, smem, tid);
 
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps descriptors in SGPRs
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps descriptors in SGPRs
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
   const int vwave = m0 + wm * G::WM;             // first vocab row of this wavefront
   const int vbase = vwave + lhi * 4;             // + mi*32 + (r/4)*8 + r%4
@@ -216,8 +219,12 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
     // where this lane's eight-entry groups go: token row, then the lane's half of a 16-entry span
     const bool store = p.zt != nullptr && (t0 + ni * 32) < zt_cols;   // tokens past the live ones are never read
     const uint32_t voff = (uint32_t)((ni * 32 + l31) * ldz2 + (vwave + lhi * 8) * 2);
+    // Rows of tokens that cannot carry a gradient (mask 0; in kStatsGrad: dloss/dlogp 0) are not
+    // written at all: the backward products know them from the dead-token bits and do not read them.
+    bool keep = true;
+    if (store) keep = MODE == kStatsGrad ? (col < p.n && p.g[col] != 0.f) : (col < p.n && p.mask[col] != 0.f);
     auto group_off = [&](int mi, int qp) {      // kOob when the lane's eight entries lie past V (V % 8 == 0)
-      return (vwave + mi * 32 + qp * 16 + lhi * 8) < p.V ? voff : kOob;
+      return (keep && (vwave + mi * 32 + qp * 16 + lhi * 8) < p.V) ? voff : kOob;
     };
 
     if (MODE == kStatsMax) {
@@ -274,13 +281,12 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
             float v[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = g.acc[mi][ni][qp * 8 + j];
-            store_rows8<true>(v, 0xffffffffu, zrs, group_off(mi, qp), (uint32_t)(mi * 32 + qp * 16) * 2);
+            store_rows8<true>(v, zrs, group_off(mi, qp), (uint32_t)(mi * 32 + qp * 16) * 2);
           }
       }
     } else if (MODE == kStatsExp) {
       float l = 0.f, s = 0.f;
       if (store) {
-        const uint32_t keep = (col < p.n && p.mask[col] != 0.f) ? 0xffffffffu : 0u;
 #pragma unroll
         for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
@@ -294,7 +300,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
               s = fmaf(e, z, s);
               v[j] = CAP ? e * (1.f - z * z * inv_cap2) : e;
             }
-            store_rows8<false>(v, keep, zrs, group_off(mi, qp), (uint32_t)(mi * 32 + qp * 16) * 2);
+            store_rows8<false>(v, zrs, group_off(mi, qp), (uint32_t)(mi * 32 + qp * 16) * 2);
           }
       } else {
 #pragma unroll
@@ -348,8 +354,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
               const float d = gneg * __builtin_amdgcn_exp2f(fmaf(z, kLog2e, -lse2));
               v[j] = CAP ? d * (1.f - z * z * inv_cap2) : d;
             }
-            store_rows8<false>(v, gneg != 0.f ? 0xffffffffu : 0u, zrs, group_off(mi, qp),
-                               (uint32_t)(mi * 32 + qp * 16) * 2);
+            store_rows8<false>(v, zrs, group_off(mi, qp), (uint32_t)(mi * 32 + qp * 16) * 2);
           }
       }
     }
@@ -372,6 +377,15 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem) {
   }
 }
 
+// A thread index that the compiler cannot trace back to threadIdx.x: inside a loop over tiles it
+// makes the per-thread address arithmetic of a tile part of that tile's code, so that none of it is
+// kept in registers across the previous tile's epilogue (where the 256 accumulators leave no room).
+MJ_DEV int opaque_tid() {
+  int t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
+}
+
 // One workgroup per tile; RESCUE: a small grid that walks the tile list, and leaves at once unless
 // the range check of the kStatsExp pass failed (state != 0).
 template <int BM, int BN, int MODE, bool RESCUE, bool CAP>
@@ -380,14 +394,15 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
   int tm, tn, split;
   if (RESCUE) {
     if (__builtin_amdgcn_readfirstlane(*p.state) == 0) return;
-    for (int item = blockIdx.x; item < map.items(); item += gridDim.x) {
-      if (map.tile(item, tm, tn, split)) logits_tile<BM, BN, MODE, CAP>(p, tm, tn, smem);
+    const int items = map.items();
+    for (int item = blockIdx.x; item < items; item += gridDim.x) {
+      if (map.tile(item, tm, tn, split)) logits_tile<BM, BN, MODE, CAP>(p, tm, tn, smem, opaque_tid());
       __syncthreads();      // the next tile's first LDS writes must not pass this tile's last reads
     }
   } else {
     if (MODE == kStatsExp && blockIdx.x == 0 && threadIdx.x == 0) *p.state = 0;
     if (!map.tile(blockIdx.x, tm, tn, split)) return;
-    logits_tile<BM, BN, MODE, CAP>(p, tm, tn, smem);
+    logits_tile<BM, BN, MODE, CAP>(p, tm, tn, smem, threadIdx.x);
   }
 }
 
@@ -417,6 +432,7 @@ struct FinalizeArgs {
   float cap;
   int* state;
   int rescue;                  // kStatsMax launched behind a kStatsExp pass: leave unless state != 0
+  uint16_t* dead;              // [n_pad / 16] dead-token bits of the chunk (bit set: no gradient), or null
 };
 
 // block = (kFinTokens tokens) x (kFinSlices slices of the partial list): few tokens per block keep a
@@ -462,74 +478,85 @@ __global__ __launch_bounds__(kFinTokens * kFinSlices) void k_finalize(FinalizeAr
   sm[ty][tx] = m; sl[ty][tx] = l; ss[ty][tx] = s; st[ty][tx] = lt;
   __syncthreads();
   if (ty != 0) return;
+  bool dead = true;
   if (t >= p.n) {
     if (p.g != nullptr && t < p.n_pad) p.g[t] = 0.f;
     if (p.ge != nullptr && t < p.n_pad) p.ge[t] = 0.f;
     if (MODE == kStatsExp && p.rs != nullptr && t < p.n_pad) p.rs[t] = 0.f;
-    return;
-  }
-  float M = 0.f, L = 0.f, S = 0.f, LT = 0.f;
-  if (MODE == kStatsExp) {
-#pragma unroll
-    for (int i = 0; i < kFinSlices; ++i) {
-      L += sl[i][tx];
-      S += ss[i][tx];
-      LT += st[i][tx];
-    }
-    // outside the window (or not finite): the sums cannot be trusted; the kStatsMax pass redoes the chunk
-    if (!(L >= kExpSumMin && L <= kExpSumMax)) *p.state = 1;
-    if (tempered && !(LT >= kExpSumMin && LT <= kExpSumMax)) *p.state = 1;
   } else {
-    M = sm[0][tx];
+    float M = 0.f, L = 0.f, S = 0.f, LT = 0.f;
+    if (MODE == kStatsExp) {
 #pragma unroll
-    for (int i = 1; i < kFinSlices; ++i) M = fmaxf(M, sm[i][tx]);
+      for (int i = 0; i < kFinSlices; ++i) {
+        L += sl[i][tx];
+        S += ss[i][tx];
+        LT += st[i][tx];
+      }
+      // outside the window (or not finite): the sums cannot be trusted; the kStatsMax pass redoes the chunk
+      if (!(L >= kExpSumMin && L <= kExpSumMax)) *p.state = 1;
+      if (tempered && !(LT >= kExpSumMin && LT <= kExpSumMax)) *p.state = 1;
+    } else {
+      M = sm[0][tx];
 #pragma unroll
-    for (int i = 0; i < kFinSlices; ++i) {
-      const float w = __expf(sm[i][tx] - M);
-      const float wt = tempered ? __expf((sm[i][tx] - M) * p.inv_t) : w;
-      L += sl[i][tx] * w;
-      S += ss[i][tx] * wt;
-      LT += st[i][tx] * wt;
+      for (int i = 1; i < kFinSlices; ++i) M = fmaxf(M, sm[i][tx]);
+#pragma unroll
+      for (int i = 0; i < kFinSlices; ++i) {
+        const float w = __expf(sm[i][tx] - M);
+        const float wt = tempered ? __expf((sm[i][tx] - M) * p.inv_t) : w;
+        L += sl[i][tx] * w;
+        S += ss[i][tx] * wt;
+        LT += st[i][tx] * wt;
+      }
+    }
+    const float lse = M + __logf(L);
+    const float zy = p.zy[t];
+    const float logp = (zy - lse) * p.inv_t;     // division after the log-softmax (:124-126)
+    p.lse[t] = lse;
+    p.logp[t] = logp;
+    // entropy of softmax(z / T): log sum e^(z/T) - sum p z / T  (reference adds 1e-9 inside the log)
+    const float H = tempered ? (M * p.inv_t + __logf(LT)) - (S / LT) * p.inv_t : lse - S / L;
+    if (p.ent != nullptr) p.ent[t] = H;
+    const float mk = p.mask[t];
+    p.eterm[t] = H * mk * p.inv_ent_cnt;
+    float ge = 0.f;
+    if (p.ge != nullptr) {
+      ge = p.ent_coef * mk * p.inv_ent_cnt * p.gscale;
+      p.ge[t] = ge;
+      p.hent[t] = H;
+    }
+    float term, g;
+    if (p.sft) {
+      term = -logp * mk * p.inv_tv;
+      g = -mk * p.inv_tv;
+    } else {
+      const float adv = p.adv[t];
+      const float ratio = p.old_logp != nullptr ? __expf(logp - p.old_logp[t]) : 1.f;
+      const float lo = 1.f - p.eps_low, hi = 1.f + p.eps_high;
+      const float clipped = fminf(fmaxf(ratio, lo), hi);
+      term = -fminf(ratio * adv, clipped * adv) * mk * p.inv_tv;
+      const bool active = (ratio >= lo && ratio <= hi) || (ratio > hi && adv < 0.f) || (ratio < lo && adv > 0.f);
+      g = active ? -mk * p.inv_tv * adv * ratio : 0.f;
+    }
+    p.term[t] = term;
+    g *= p.gscale * p.inv_t;                     // dlogp/dz = (onehot - softmax(z)) / T
+    if (p.g != nullptr) p.g[t] = g;
+    // a row takes part in the backward products unless its whole gradient is zero; a masked token is
+    // always dead (its row of the 16-bit matrix was not even written), whatever g evaluates to
+    dead = mk == 0.f || (!(g != 0.f) && !(ge != 0.f));
+    if (MODE == kStatsExp && p.rs != nullptr) {
+      // dZ[t, v] = g (onehot - e_v / L) cap'_v = (-g / L) (E[t, v] - onehot * L * cap'_y)
+      p.rs[t] = -g / L;
+      if (mk != 0.f) {                           // rows of masked tokens do not exist
+        const int y = clamp_target(p.targets[t], p.V);
+        const float capf = p.cap > 0.f ? 1.f - (zy / p.cap) * (zy / p.cap) : 1.f;
+        p.zt[(int64_t)t * p.ld_z + y] = f32_to_bf16((__builtin_amdgcn_exp2f(zy * kLog2e) - L) * capf);
+      }
     }
   }
-  const float lse = M + __logf(L);
-  const float zy = p.zy[t];
-  const float logp = (zy - lse) * p.inv_t;     // division after the log-softmax (:124-126)
-  p.lse[t] = lse;
-  p.logp[t] = logp;
-  // entropy of softmax(z / T): log sum e^(z/T) - sum p z / T  (reference adds 1e-9 inside the log)
-  const float H = tempered ? (M * p.inv_t + __logf(LT)) - (S / LT) * p.inv_t : lse - S / L;
-  if (p.ent != nullptr) p.ent[t] = H;
-  const float mk = p.mask[t];
-  p.eterm[t] = H * mk * p.inv_ent_cnt;
-  if (p.ge != nullptr) {
-    p.ge[t] = p.ent_coef * mk * p.inv_ent_cnt * p.gscale;
-    p.hent[t] = H;
-  }
-  float term, g;
-  if (p.sft) {
-    term = -logp * mk * p.inv_tv;
-    g = -mk * p.inv_tv;
-  } else {
-    const float adv = p.adv[t];
-    const float ratio = p.old_logp != nullptr ? __expf(logp - p.old_logp[t]) : 1.f;
-    const float lo = 1.f - p.eps_low, hi = 1.f + p.eps_high;
-    const float clipped = fminf(fmaxf(ratio, lo), hi);
-    term = -fminf(ratio * adv, clipped * adv) * mk * p.inv_tv;
-    const bool active = (ratio >= lo && ratio <= hi) || (ratio > hi && adv < 0.f) || (ratio < lo && adv > 0.f);
-    g = active ? -mk * p.inv_tv * adv * ratio : 0.f;
-  }
-  p.term[t] = term;
-  g *= p.gscale * p.inv_t;                     // dlogp/dz = (onehot - softmax(z)) / T
-  if (p.g != nullptr) p.g[t] = g;
-  if (MODE == kStatsExp && p.rs != nullptr) {
-    // dZ[t, v] = g (onehot - e_v / L) cap'_v = (-g / L) (E[t, v] - onehot * L * cap'_y)
-    p.rs[t] = -g / L;
-    if (mk != 0.f) {                           // masked tokens keep their zero row
-      const int y = clamp_target(p.targets[t], p.V);
-      const float capf = p.cap > 0.f ? 1.f - (zy / p.cap) * (zy / p.cap) : 1.f;
-      p.zt[(int64_t)t * p.ld_z + y] = f32_to_bf16((__builtin_amdgcn_exp2f(zy * kLog2e) - L) * capf);
-    }
+  if (p.dead != nullptr) {
+    // the 16 finalising threads are lanes 0..15 of the block's first wavefront
+    const uint64_t bits = __ballot(dead);
+    if (tx == 0) p.dead[blockIdx.x] = (uint16_t)bits;
   }
 }
 
@@ -554,10 +581,10 @@ __global__ __launch_bounds__(256) void k_scale_hidden(const uint16_t* hid, int64
 __global__ __launch_bounds__(256) void k_coeff_from_saved(const float* logp, const float* old_logp,
                                                           const float* adv, const float* mask, int n,
                                                           int n_pad, float eps_low, float eps_high,
-                                                          float inv_tv, float gscale, int sft, float* g) {
-  // gscale carries 1 / temperature as well (see k_finalize)
+                                                          float inv_tv, float gscale, int sft, float* g,
+                                                          uint64_t* dead) {
+  // gscale carries 1 / temperature as well (see k_finalize); n_pad is a multiple of 256 = the block
   const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t >= n_pad) return;
   float out = 0.f;
   if (t < n) {
     const float mk = mask[t];
@@ -571,7 +598,10 @@ __global__ __launch_bounds__(256) void k_coeff_from_saved(const float* logp, con
       out = active ? -mk * inv_tv * a * ratio : 0.f;
     }
   }
-  g[t] = out * gscale;
+  out *= gscale;
+  g[t] = out;
+  const uint64_t bits = __ballot(!(out != 0.f));      // the epilogue stores the rows with g != 0
+  if ((threadIdx.x & 63) == 0) dead[t >> 6] = bits;
 }
 
 // kStatsGrad: the sampled token's entry of dZ, g (1 - p_y) cap'_y, replaces the -g p_y cap'_y the
@@ -622,6 +652,7 @@ struct DzArgs {
   const float *lse, *g;    // chunk-local (lse valid for t < n, g for t < n_pad)
   const float *ge, *hent;  // chunk-local entropy-bonus coefficient and H_t, or null
   const int32_t* targets;  // chunk origin
+  const float* mask;       // chunk origin
   int V, n;
   float cap;
   const int* n_live;   // see live_pad
@@ -642,11 +673,12 @@ __global__ __launch_bounds__(256) void k_dz(DzArgs p) {
     const float lse = p.lse[t] * kLog2e, g = p.g[t];
     const float ge = bonus ? p.ge[t] : 0.f, hent = bonus ? p.hent[t] : 0.f;
     const int y = clamp_target(p.targets[t], p.V);
-    const bool dead = !(g != 0.f) && !(ge != 0.f);   // masked token: exactly zero, whatever z holds
+    // a token without a gradient: the backward products do not read its row (dead-token bits)
+    if (p.mask[t] == 0.f || (!(g != 0.f) && !(ge != 0.f))) continue;
     uint16_t* row = p.zt + (int64_t)t * p.ld_z;
     for (int v0 = threadIdx.x * 8; v0 < p.V; v0 += 256 * 8) {
       u32x4 out = {0u, 0u, 0u, 0u};
-      if (!dead) {
+      {
         const u32x4 in = *(const u32x4*)(row + v0);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -682,11 +714,12 @@ struct DhArgs {
   const float* rs;    // [n_pad] row scale, applied when state == 0
   const int* state;
   const float *dv, *wv;   // value head (PPO critic): d_hidden[t, :] += dv[t] * wv[:]; both null = none
+  const uint64_t* dead;   // [n_pad / 64] dead-token bits of the chunk
 };
 
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
-  using G = GemmTN<BM, BN, kRowK, kRowK>;
+  using G = GemmTN<BM, BN, kRowK, kRowK, 1, true, false>;   // rows of dead tokens are not fetched
   extern __shared__ __attribute__((aligned(16))) char smem[];
   // Only token tiles that hold live tokens are walked: the tile list is rebuilt for that many
   // rows of tiles, so that the live work spreads evenly over the XCDs (ids past its end leave).
@@ -698,7 +731,7 @@ __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
   const int klen = min(p.V - k0, p.k_per_split);
   G g;
   g.run(p.dzt + (int64_t)m0 * p.ld_z + k0, p.n - m0, p.ld_z, p.w + (int64_t)n0 * p.ld_w + k0, p.H - n0, p.ld_w,
-        klen, smem);
+        klen, smem, threadIdx.x, p.dead + m0 / 64);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps descriptors in SGPRs
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
@@ -777,6 +810,7 @@ struct DwArgs {
   const int* n_live;   // see live_pad
   int c0;
   const int* state;
+  const uint64_t* dead;   // [n_pad / 64] dead-token bits of the chunk
 };
 
 // Tile of dW^T: rows = vocab (MFMA row direction), columns = hidden (lanes).  A lane's four
@@ -786,7 +820,9 @@ struct DwArgs {
 // consecutive entries of one row, and an accumulating call adds in fp32 and rounds once.
 template <int BM, int BN, bool BF16OUT>
 __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
-  using G = GemmTN<BM, BN, kKRow, kKRow, 2>;   // two slices in flight: measured 2-3% faster here, not in the other products
+  // two slices in flight: measured 2-3% faster here, not in the other products; the token rows of
+  // dead tokens (k-rows of both operands) are not fetched
+  using G = GemmTN<BM, BN, kKRow, kKRow, 2, true, true>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   int tm, tn, split;
   if (!map.tile(blockIdx.x, tm, tn, split)) return;
@@ -796,7 +832,7 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
   const bool scaled = __builtin_amdgcn_readfirstlane(*p.state) == 0;
   const __bf16* tok = scaled ? p.hs : p.hid;
   const int64_t ld_tok = scaled ? (int64_t)p.H : p.ld_hid;
-  g.run(p.dzt + m0, p.V - m0, p.ld_z, tok + n0, p.H - n0, ld_tok, kn, smem);
+  g.run(p.dzt + m0, p.V - m0, p.ld_z, tok + n0, p.H - n0, ld_tok, kn, smem, threadIdx.x, p.dead, p.dead);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps descriptors in SGPRs
   const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
@@ -843,7 +879,7 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
               v[2 * j + 1] += __uint_as_float(w[j] & 0xffff0000u);
             }
           }
-          store_rows8<false>(v, 0xffffffffu, rs, (vv + lhi * 8) < vleft ? lane_off : kOob, (uint32_t)vv * 2);
+          store_rows8<false>(v, rs, (vv + lhi * 8) < vleft ? lane_off : kOob, (uint32_t)vv * 2);
         }
     }
     return;

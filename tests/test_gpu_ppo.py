@@ -36,12 +36,14 @@ def _batch(seed, b, l, h, v, vocab_in=50):
 
 
 def _run_case(seed, b, l, h, v, *, old_noise=0.0, returns=False, old_values=False, adv_per_seq=False,
-              tvtc=None, chunk_tokens=None, **hyper):
+              tvtc=None, chunk_tokens=None, zero_adv_seqs=(), **hyper):
     import mllm_jax_amd as M
     dev = torch.device("cuda:0")
     ids, emb, pos, w, wv, bv, labels, adv = _batch(seed, b, l, h, v)
     g = torch.Generator().manual_seed(seed + 1)
     t = l - 1
+    for s_ in zero_adv_seqs:
+        adv[s_] = 0.0                       # a group whose rewards are all equal: advantages exactly 0
     hidden_cpu = (emb[ids].float() + pos[None].float()).to(torch.bfloat16)        # [b,l,h]
     hid_flat = hidden_cpu[:, :-1].reshape(b * t, h).float().numpy()
     y = ids[:, 1:].reshape(-1).numpy()
@@ -137,6 +139,17 @@ def test_value_head_gradient_joins_d_hidden_in_the_product(splits):
 def test_value_head_with_skip_masked_and_chunks():
     _run_case(9, 6, 97, 64, 776, returns=True, old_values=True, old_noise=0.1, chunk_tokens=256, skip_masked=True)
     _run_case(10, 3, 41, 64, 520, skip_masked=True, entropy_coef=0.02, returns=True)
+
+
+def test_skip_masked_keeps_the_critic_gradient_of_zero_advantage_tokens():
+    """Advantage exactly 0 (every reward of a GRPO group equal) zeroes the policy gradient of a token
+    but not the critic's: with returns given, d value_loss / d value_pred = 2 (v - R) reaches d_hidden
+    through dv[t] * value_w, so such tokens must stay in the compacted batch."""
+    out, ref = _run_case(11, 4, 65, 64, 776, returns=True, old_values=True, old_noise=0.1, skip_masked=True,
+                         zero_adv_seqs=(1, 2))
+    rows = np.abs(ref["d_hidden"].reshape(4, 64, 64)[1]).sum(-1)
+    assert (rows > 0).any(), "the case must hold zero-advantage tokens with a critic gradient"
+    _run_case(12, 4, 33, 64, 520, returns=True, skip_masked=True, zero_adv_seqs=(0, 1, 2, 3), chunk_tokens=256)
 
 
 def test_value_method_and_no_grad_call_match_the_oracle():
