@@ -118,9 +118,9 @@ int mj_grpo_forward(const MjGrpoDesc* desc, const void* hidden, const void* lm_h
  * does not fit even with 256-token chunks (12 bytes per token plus 6 * ceil(V/256) * 4 bytes per
  * token of a chunk) are refused with MJ_GRPO_ERR_WORKSPACE.  All calls on one device share the
  * array: calls that overlap on a device (two streams, two threads) race; serialise them.  Outputs
- * are those of mj_grpo_forward bit for bit.  The first call on a device looks the array's address
- * up (hipGetSymbolAddress) and raises the kernels' LDS limit (hipFuncSetAttribute): make one call
- * outside stream capture before capturing others. */
+ * are those of mj_grpo_forward bit for bit.  The first call on a device (from any thread) looks the
+ * array's address up (hipGetSymbolAddress) and raises the kernels' LDS limit (hipFuncSetAttribute):
+ * make one call per device outside stream capture before capturing others. */
 #define MJ_GRPO_NOALLOC_SCRATCH_BYTES (32u << 20)
 int mj_grpo_forward_noalloc(const MjGrpoDesc* desc, const void* hidden, const void* lm_head,
                             const int32_t* targets, const float* old_logp, const float* advantages,
@@ -140,6 +140,17 @@ int mj_grpo_forward_backward(const MjGrpoDesc* desc, const void* hidden, const v
                              float* lse, float* token_entropy, float* loss, void* d_hidden,
                              void* d_lm_head, void* workspace, size_t workspace_bytes,
                              void* stream);
+
+/* Upstream gradient that is only known on the device.  The reference differentiates the loss itself
+ * (jax.value_and_grad, plugins/training/update/train_step.py:15-24: upstream gradient 1, which is what
+ * grad_loss_scale = 1 gives); a caller whose autodiff hands it d(total)/d(loss) as a device scalar
+ * after the fused pass has run (torch.autograd) applies it here: d_hidden[n, ld_hidden] bf16 and
+ * d_lm_head[h, ld_w] (float32, or bf16 when d_lm_head_bf16 != 0) are multiplied in place by *scale.
+ * When *scale == 1 every workgroup leaves at once: no pass over either matrix, no host
+ * synchronisation.  Either pointer may be NULL (skipped).  Padding columns past h / v are untouched. */
+int mj_grpo_scale_gradients(void* d_hidden, int64_t n, int64_t h, int64_t ld_hidden, void* d_lm_head,
+                            int64_t lm_head_rows, int64_t v, int64_t ld_w, int d_lm_head_bf16,
+                            const float* scale, void* stream);
 
 /* The two per-sequence entropy entries of the reference's return dict
  * (MLLM_JAX/train_modules/__init__.py:141-157) from the per-token entropies of a forward:
@@ -222,12 +233,14 @@ int mj_grpo_gae(const float* rewards, const float* values, const float* completi
                 float* advantages, float* returns, int64_t b, int64_t t, float gamma, float gae_lambda,
                 int normalize, float eps, float clip_range, void* stream);
 
-/* Optional per-kernel timing (bench and profiling; no counterpart in the reference, whose only
- * timers are wall-clock phase timers, plugins/training/runner/grpo_gsm8k.py:615-792).
- * Between begin and end every kernel launch of the entry points above is bracketed by a pair of
- * HIP events recorded on the caller's stream.  mj_grpo_profile_end waits for them and returns,
- * per kernel id, the summed duration in milliseconds and the number of launches.  Process-wide
- * and not thread-safe: use from one thread. */
+/* Launch tracing.  The reference's observability of this path is a set of wall-clock phase timers
+ * around the update (plugins/training/runner/grpo_gsm8k.py:615-792, printed under
+ * PRINT_TRAIN_TIME_BREAKDOWN); here a caller can watch the individual kernels.  While a callback is
+ * set, every kernel launch of the entry points above is bracketed by two calls of it on the calling
+ * thread: phase 0 just before the launch is enqueued on `stream`, phase 1 just after (the three
+ * launches of the running-maximum rescue pass count as one, MJ_GRPO_K_RESCUE).  The callback may
+ * record events on `stream`; it must not synchronise or enqueue work that the kernels depend on.
+ * fn == NULL switches tracing off.  Process-wide and not thread-safe: set it while no call runs. */
 enum {
   MJ_GRPO_K_LOGITS_STATS = 0,
   MJ_GRPO_K_FINALIZE = 1,
@@ -237,20 +250,11 @@ enum {
   MJ_GRPO_K_DW = 5,
   MJ_GRPO_K_REDUCE_LOSS = 6,
   MJ_GRPO_K_SCALE_HIDDEN = 7,
-  MJ_GRPO_K_RESCUE = 8,       /* the three launches of the running-maximum rescue pass together */
+  MJ_GRPO_K_RESCUE = 8,
   MJ_GRPO_K_COUNT = 9
 };
-int mj_grpo_profile_begin(int max_launches);
-int mj_grpo_profile_end(double* total_ms /* [MJ_GRPO_K_COUNT] */, int* launches /* [MJ_GRPO_K_COUNT] */);
-
-/* Measurement support (no counterpart in the reference): an MFMA-only loop with the register tile
- * of the product kernels (4 wavefronts x 16 blocks of v_mfma_f32_32x32x16_bf16 per workgroup, no
- * memory traffic while it runs).  operands: 1 MiB of bf16 data on the device (what the multipliers
- * see: random values or zeros); out: workgroups * 256 floats; *flop receives the flop executed.
- * Timed by the caller with events on `stream`; shows what the matrix cores sustain under the
- * GPU's power cap for a given operand data pattern. */
-int mj_grpo_probe_mfma(const void* operands, float* out, int workgroups, int iters, double* flop,
-                       void* stream);
+typedef void (*MjGrpoTraceFn)(void* user, int kernel_id, int phase, void* stream);
+int mj_grpo_set_trace(MjGrpoTraceFn fn, void* user);
 
 #ifdef __cplusplus
 }

@@ -29,7 +29,8 @@ int mj_sample_logits(const void* hidden, int64_t ld_hidden, const void* lm_head,
                      float* logits, int64_t ld_logits, int64_t b, int64_t h, int64_t vocab,
                      float softcap, void* stream);
 
-/* Per row: the k (<= 64) largest of logits * (1/t) in descending order (equal values: lower index
+/* Per row: the k (<= 64) largest of logits / t (a division, as the reference's `logits / t`,
+ * MLLM_JAX/sample/sanple_utils.py:37) in descending order (equal values: lower index
  * first, as jax.lax.top_k), then token = top_idx[argmax_j(top_val[j] + noise[j])] (first maximum
  * on ties, as jnp.argmax).  noise == NULL draws greedily (the largest logit).  top_idx / top_val
  * ([b, k]) may be NULL. */

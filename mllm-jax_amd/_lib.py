@@ -17,8 +17,8 @@ FLAG_SKIP_MASKED = 1 << 2
 FLAG_DW_BF16 = 1 << 3
 
 EXPORTS = ("mj_grpo_version", "mj_grpo_last_error", "mj_grpo_workspace_bytes", "mj_grpo_forward",
-           "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_forward_noalloc", "mj_grpo_probe_mfma", "mj_grpo_forward_backward_value",
-           "mj_grpo_value_workspace_bytes", "mj_value_head_forward", "mj_grpo_sequence_entropy", "mj_grpo_profile_begin", "mj_grpo_profile_end",
+           "mj_grpo_forward_backward", "mj_grpo_backward", "mj_grpo_forward_noalloc", "mj_grpo_set_trace", "mj_grpo_forward_backward_value",
+           "mj_grpo_value_workspace_bytes", "mj_value_head_forward", "mj_grpo_sequence_entropy", "mj_grpo_scale_gradients",
            "mj_grpo_group_advantages", "mj_grpo_advantages", "mj_grpo_gae", "mj_rmsnorm_forward", "mj_sample_logits", "mj_sample_top_k", "mj_rmsnorm_workspace_bytes", "mj_rmsnorm_backward")
 
 KERNEL_NAMES = ("k_logits_stats", "k_finalize", "k_dz", "k_dhidden", "k_dhidden_reduce", "k_dw",
@@ -69,7 +69,9 @@ def load() -> C.CDLL:
     lib.mj_grpo_workspace_bytes.argtypes = [dp, C.POINTER(sz), C.POINTER(sz)]
     lib.mj_grpo_forward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp, sz, vp]
     lib.mj_grpo_forward_noalloc.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp]
-    lib.mj_grpo_probe_mfma.argtypes = [vp, fp, C.c_int, C.c_int, C.POINTER(C.c_double), vp]
+    lib.mj_grpo_set_trace.argtypes = [vp, vp]
+    lib.mj_grpo_scale_gradients.argtypes = [vp, C.c_int64, C.c_int64, C.c_int64, vp, C.c_int64, C.c_int64, C.c_int64,
+                                            C.c_int, fp, vp]
     lib.mj_grpo_forward_backward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp, fp, vp, sz, vp]
     lib.mj_grpo_forward_backward_value.argtypes = [dp, C.POINTER(MjPpoValue), vp, vp, ip, fp, fp, fp, fp, fp, fp, fp, vp, fp,
                                                    vp, sz, vp]
@@ -77,8 +79,6 @@ def load() -> C.CDLL:
     lib.mj_value_head_forward.argtypes = [vp, C.c_int64, fp, fp, fp, C.c_int64, C.c_int64, vp]
     lib.mj_grpo_sequence_entropy.argtypes = [fp, fp, C.c_int64, C.c_int64, fp, fp, vp]
     lib.mj_grpo_backward.argtypes = [dp, vp, vp, ip, fp, fp, fp, fp, fp, vp, fp, vp, sz, vp]
-    lib.mj_grpo_profile_begin.argtypes = [C.c_int]
-    lib.mj_grpo_profile_end.argtypes = [C.POINTER(C.c_double), C.POINTER(C.c_int)]
     i64, f32 = C.c_int64, C.c_float
     lib.mj_grpo_group_advantages.argtypes = [fp, ip, fp, i64, f32, vp]
     lib.mj_grpo_advantages.argtypes = [C.c_int, fp, ip, fp, i64, f32, f32, C.c_int, f32, vp]
@@ -109,15 +109,3 @@ def value_workspace_bytes(desc: MjGrpoDesc) -> int:
     b = C.c_size_t(0)
     check(load().mj_grpo_value_workspace_bytes(C.byref(desc), C.byref(b)))
     return b.value
-
-
-def profile_begin(max_launches: int = 4096) -> None:
-    check(load().mj_grpo_profile_begin(max_launches))
-
-
-def profile_end() -> dict:
-    """{kernel name: (total_ms, launches)} since profile_begin."""
-    n = len(KERNEL_NAMES)
-    ms, cnt = (C.c_double * n)(), (C.c_int * n)()
-    check(load().mj_grpo_profile_end(ms, cnt))
-    return {KERNEL_NAMES[i]: (ms[i], cnt[i]) for i in range(n)}

@@ -1,7 +1,9 @@
-"""Builds libmj_grpo.so (the C-ABI library of HIP kernels) for gfx950 with hipcc.
+"""Builds libmj_grpo.so (the C-ABI library of HIP kernels) and libmj_grpo_bench.so (bench.py's
+measurement support: event timing behind the launch-trace hook, the MFMA-only probe) for gfx950
+with hipcc.
 
 `python -m mllm_jax_amd.build` compiles in-tree; tests, the smoke entry and the bench
-load the built library and never compile on a GPU box.
+load the built libraries and never compile on a GPU box.
 """
 from __future__ import annotations
 
@@ -13,6 +15,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 SRC = os.path.join(HERE, "csrc", "mj_grpo.hip")
 LIB = os.path.join(HERE, "libmj_grpo.so")
+BENCH_SRC = os.path.join(HERE, "csrc", "mj_bench.hip")
+BENCH_LIB = os.path.join(HERE, "libmj_grpo_bench.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -29,7 +33,12 @@ def hipcc_path() -> str:
 
 
 def build(verbose: bool = True) -> str:
-    cmd = [hipcc_path(), *HIPCC_FLAGS, SRC, "-o", LIB + ".tmp"]
+    _compile(BENCH_SRC, BENCH_LIB, verbose)
+    return _compile(SRC, LIB, verbose)
+
+
+def _compile(src: str, lib: str, verbose: bool) -> str:
+    cmd = [hipcc_path(), *HIPCC_FLAGS, src, "-o", lib + ".tmp"]
     if verbose:
         print("+", " ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -40,9 +49,9 @@ def build(verbose: bool = True) -> str:
     if verbose and err.strip():
         print(err, file=sys.stderr)
     import ctypes
-    ctypes.CDLL(LIB + ".tmp")          # an unresolved symbol must fail the build, not the first call
-    os.replace(LIB + ".tmp", LIB)
-    return LIB
+    ctypes.CDLL(lib + ".tmp")          # an unresolved symbol must fail the build, not the first call
+    os.replace(lib + ".tmp", lib)
+    return lib
 
 
 if __name__ == "__main__":

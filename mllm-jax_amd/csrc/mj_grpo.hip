@@ -14,167 +14,64 @@
 
 #include "mj_grpo_kernels.hpp"
 #include "mj_norm_kernels.hpp"
-#include "mj_probe_kernels.hpp"
+#include "plan.hpp"
 
 namespace {
 
-thread_local char g_err[512] = "";
+using namespace mj::host;
+static_assert(mj::kValueRows == mj::host::kValueRows, "the plan sizes the value head's partial rows");
 
-int fail(int code, const char* fmt, ...) {
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(g_err, sizeof(g_err), fmt, ap);
-  va_end(ap);
-  return code;
-}
-
-// ---- optional per-kernel timing with HIP events on the caller's stream (bench / profiling only)
-struct Profiler {
-  bool on = false;
-  hipEvent_t* ev = nullptr;
-  int* kid = nullptr;
-  int cap = 0, used = 0;   // event pairs
-} g_prof;
+// ---- launch tracing (mj_grpo_set_trace): a callback before and after every kernel launch
+struct Trace {
+  MjGrpoTraceFn fn = nullptr;
+  void* user = nullptr;
+} g_trace;
 
 struct Timed {
   hipStream_t st;
-  bool active;
-  Timed(int kernel_id, hipStream_t s) : st(s), active(g_prof.on && g_prof.used < g_prof.cap) {
-    if (active) {
-      g_prof.kid[g_prof.used] = kernel_id;
-      (void)hipEventRecord(g_prof.ev[2 * g_prof.used], st);
-    }
+  int id;
+  MjGrpoTraceFn fn;
+  void* user;
+  Timed(int kernel_id, hipStream_t s) : st(s), id(kernel_id), fn(g_trace.fn), user(g_trace.user) {
+    if (fn) fn(user, id, 0, (void*)st);
   }
   ~Timed() {
-    if (active) {
-      (void)hipEventRecord(g_prof.ev[2 * g_prof.used + 1], st);
-      ++g_prof.used;
-    }
+    if (fn) fn(user, id, 1, (void*)st);
   }
 };
-
-constexpr int BM = 256, BN = 256;          // tile of all three contractions
-constexpr int64_t kDefaultChunk = 16384;   // tokens whose logits live in the workspace at once
-constexpr int kRescueGrid = 256;           // workgroups of the rescue pass (one per CU)
-
-inline int64_t rup(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
-
-struct Plan {
-  int64_t N, H, V, chunk, n_pad, ld_z, parts;
-  int dh_splits;          // vocab splits of the dHidden product (1 = none)
-  int64_t dh_k_per_split;
-  // byte offsets into the workspace
-  size_t zy, term, eterm, pm, pl, ps, plt, g, ge, hent, state, rs, dead, hs, zt, part, total_fwd, total_bwd;
-  // token compaction (MJ_GRPO_FLAG_SKIP_MASKED): slot-order copies of the inputs and outputs
-  bool compact;
-  size_t perm, n_live, hid_p, tgt_p, fin_p[5], fout_p[3], dh_p;
-  // value head (mj_grpo_forward_backward_value): laid out behind total_bwd
-  size_t v_term, v_dv, v_dv_p, v_part, total_value;
-};
-
-// Splits of the dHidden product over the vocab: its (n/256) x (H/256) tiles rarely fill the 256
-// CUs in whole rounds, so K = V is cut into the fewest pieces (<= 32) that waste < 4% of a round.
-int pick_splits(int64_t tiles) {
-  int best = 1;
-  double best_eff = 0.0;
-  for (int s = 1; s <= 32; ++s) {
-    const int64_t items = tiles * s, rounds = (items + 255) / 256;
-    const double eff = (double)items / (double)(rounds * 256);
-    if (eff > best_eff + 1e-9) { best_eff = eff; best = s; }
-    if (eff >= 0.96) return s;
-  }
-  return best;
-}
-
-int make_plan(const MjGrpoDesc* d, Plan* p) {
-  if (d == nullptr) return fail(MJ_GRPO_ERR_NULL, "desc is NULL");
-  if (d->n_tokens <= 0 || d->hidden <= 0 || d->vocab <= 0)
-    return fail(MJ_GRPO_ERR_SHAPE, "n_tokens/hidden/vocab must be positive (got %lld/%lld/%lld)",
-                (long long)d->n_tokens, (long long)d->hidden, (long long)d->vocab);
-  // 256 rows of any operand or output must fit one 2 GiB buffer descriptor
-  if (d->n_tokens > (1ll << 30) || d->hidden > (1 << 20) || d->vocab > (1 << 21) || d->ld_hidden > (1 << 20) ||
-      d->ld_w > (1 << 21) || d->chunk_tokens > (1 << 20))
-    return fail(MJ_GRPO_ERR_SHAPE, "shape too large (hidden, ld_hidden <= 2^20; vocab, ld_w <= 2^21; chunk_tokens <= 2^20)");
-  if (d->ld_hidden < d->hidden || d->ld_w < d->vocab)
-    return fail(MJ_GRPO_ERR_SHAPE, "leading dimension smaller than row length");
-  if (d->hidden % 8 || d->vocab % 8 || d->ld_hidden % 8 || d->ld_w % 8)
-    return fail(MJ_GRPO_ERR_ALIGN, "hidden, vocab, ld_hidden and ld_w must be multiples of 8");
-  if (!(d->temperature > 0.f) || !isfinite(d->temperature))
-    return fail(MJ_GRPO_ERR_UNSUPPORTED, "temperature must be positive and finite (got %g)", (double)d->temperature);
-  if (d->temperature != 1.0f && d->entropy_coef != 0.f)
-    return fail(MJ_GRPO_ERR_UNSUPPORTED, "an entropy bonus needs temperature 1 (got %g)", (double)d->temperature);
-  if (d->softcap < 0.f || !isfinite(d->softcap)) return fail(MJ_GRPO_ERR_UNSUPPORTED, "softcap must be >= 0");
-  if (d->chunk_tokens < 0) return fail(MJ_GRPO_ERR_SHAPE, "chunk_tokens must be >= 0");
-  if (d->flags & ~(uint32_t)(MJ_GRPO_FLAG_DW_ACCUMULATE | MJ_GRPO_FLAG_SFT | MJ_GRPO_FLAG_SKIP_MASKED | MJ_GRPO_FLAG_DW_BF16))
-    return fail(MJ_GRPO_ERR_UNSUPPORTED, "unknown bits in flags (0x%x)", d->flags);
-  if (!isfinite(d->inv_total_valid_tokens)) return fail(MJ_GRPO_ERR_SHAPE, "inv_total_valid_tokens not finite");
-  if (!isfinite(d->entropy_coef) || !isfinite(d->inv_entropy_count) || d->inv_entropy_count < 0.f)
-    return fail(MJ_GRPO_ERR_SHAPE, "entropy_coef / inv_entropy_count not finite");
-  p->N = d->n_tokens; p->H = d->hidden; p->V = d->vocab;
-  int64_t chunk = d->chunk_tokens > 0 ? d->chunk_tokens : kDefaultChunk;
-  chunk = rup(chunk, 256);
-  if (chunk > p->N) chunk = p->N;
-  p->chunk = chunk;
-  p->n_pad = rup(chunk, 256);
-  p->ld_z = p->V;               // rows of the 16-bit matrix: V % 8 == 0 keeps them 16-byte aligned
-  p->parts = 2 * ((p->V + BM - 1) / BM);
-  if (d->dhidden_splits > 32) return fail(MJ_GRPO_ERR_SHAPE, "dhidden_splits must be <= 32 (got %u)", d->dhidden_splits);
-  p->dh_splits = d->dhidden_splits ? (int)d->dhidden_splits : pick_splits((p->n_pad / BM) * ((p->H + BN - 1) / BN));
-  p->dh_k_per_split = rup((p->V + p->dh_splits - 1) / p->dh_splits, 64);
-  size_t o = 0;
-  auto take = [&](size_t bytes) { size_t at = o; o = (size_t)rup((int64_t)(o + bytes), 256); return at; };
-  p->zy = take((size_t)p->N * 4);
-  p->term = take((size_t)p->N * 4);
-  p->eterm = take((size_t)p->N * 4);
-  p->pm = take((size_t)p->parts * p->n_pad * 4);
-  p->pl = take((size_t)p->parts * p->n_pad * 4);
-  p->ps = take((size_t)p->parts * p->n_pad * 4);
-  p->plt = take(d->temperature != 1.0f ? (size_t)p->parts * p->n_pad * 4 : 0);
-  p->g = take((size_t)p->n_pad * 4);
-  p->ge = take((size_t)p->n_pad * 4);
-  p->hent = take((size_t)p->n_pad * 4);
-  p->state = take(256);
-  p->compact = (d->flags & MJ_GRPO_FLAG_SKIP_MASKED) != 0;
-  if (p->compact) {
-    p->perm = take((size_t)p->N * 4);
-    p->n_live = take(256);
-    p->hid_p = take((size_t)p->N * p->H * 2);
-    p->tgt_p = take((size_t)p->N * 4);
-    for (auto& f : p->fin_p) f = take((size_t)p->N * 4);
-    for (auto& f : p->fout_p) f = take((size_t)p->N * 4);
-  }
-  p->total_fwd = o;
-  p->dh_p = take(p->compact ? (size_t)p->N * p->H * 2 : 0);
-  p->rs = take((size_t)p->n_pad * 4);
-  p->dead = take((size_t)p->n_pad / 8);     // one bit per token of a chunk
-  p->hs = take((size_t)p->n_pad * p->H * 2);
-  p->zt = take((size_t)p->n_pad * p->ld_z * 2);
-  p->part = take(p->dh_splits > 1 ? (size_t)p->dh_splits * p->n_pad * p->H * 4 : 0);
-  p->total_bwd = o;
-  p->v_term = take((size_t)p->N * 4);
-  p->v_dv = take((size_t)rup(p->N, 256) * 4);
-  p->v_dv_p = take(p->compact ? (size_t)rup(p->N, 256) * 4 : 0);
-  p->v_part = take((size_t)((p->N + mj::kValueRows - 1) / mj::kValueRows) * p->H * 4);
-  p->total_value = o;
-  return MJ_GRPO_OK;
-}
 
 bool misaligned(const void* p) { return ((uintptr_t)p & 15u) != 0; }
 
-// Raises the dynamic LDS limit of a tile kernel (128 KB > the 64 KB default) once per device and
-// thread; the attribute belongs to the function on the current device.
+// Raises the dynamic LDS limit of a tile kernel (128 KB > the 64 KB default).  The attribute belongs to
+// the function on a device: it is set on the first call that launches that kernel on that device,
+// whatever thread makes it (one process-wide table under a mutex), never again afterwards.
+constexpr int kMaxDevices = 64;
+constexpr int kMaxTileKernels = 32;       // tile-kernel instantiations in this file: 15
+struct LdsDone {
+  const void* fn;
+  bool dev[kMaxDevices];
+};
+std::mutex g_lds_mutex;
+LdsDone g_lds_done[kMaxTileKernels] = {};
+
 template <typename K>
 int enable_lds(K kernel) {
-  struct Done { const void* fn; int dev; };
-  static thread_local Done done[32] = {};
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
-  for (auto& d : done) if (d.fn == (const void*)kernel && d.dev == dev) return MJ_GRPO_OK;
+  if (dev < 0 || dev >= kMaxDevices) return fail(MJ_GRPO_ERR_UNSUPPORTED, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_lds_mutex);
+  LdsDone* slot = nullptr;
+  for (auto& d : g_lds_done) {
+    if (d.fn == (const void*)kernel || d.fn == nullptr) { slot = &d; break; }
+  }
+  if (slot == nullptr) return fail(MJ_GRPO_ERR_UNSUPPORTED, "internal: more tile kernels than table slots");
+  if (slot->fn == (const void*)kernel && slot->dev[dev]) return MJ_GRPO_OK;
   e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                           mj::GemmTN<BM, BN>::kLdsBytes);
   if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-  for (auto& d : done) if (d.fn == nullptr) { d.fn = (const void*)kernel; d.dev = dev; break; }
+  slot->fn = (const void*)kernel;
+  slot->dev[dev] = true;
   return MJ_GRPO_OK;
 }
 
@@ -476,47 +373,12 @@ extern "C" {
 
 int mj_grpo_version(void) { return 300; }   // 0.3.0: MJ_GRPO_FLAG_DW_BF16, d_lm_head as void*
 
-const char* mj_grpo_last_error(void) { return g_err; }
+const char* mj_grpo_last_error(void) { return mj::host::g_err; }
 
-int mj_grpo_profile_begin(int max_launches) {
-  if (g_prof.on) return fail(MJ_GRPO_ERR_UNSUPPORTED, "profiling already on");
-  if (max_launches <= 0 || max_launches > (1 << 16)) return fail(MJ_GRPO_ERR_SHAPE, "max_launches out of range");
-  g_prof.ev = new (std::nothrow) hipEvent_t[2 * (size_t)max_launches];
-  g_prof.kid = new (std::nothrow) int[max_launches];
-  hipError_t e = (g_prof.ev && g_prof.kid) ? hipSuccess : hipErrorOutOfMemory;
-  int made = 0;
-  for (; e == hipSuccess && made < 2 * max_launches; ++made) e = hipEventCreate(&g_prof.ev[made]);
-  if (e != hipSuccess) {   // undo the partial set-up: nothing stays allocated after a failure
-    for (int i = 0; i + 1 < made; ++i) (void)hipEventDestroy(g_prof.ev[i]);
-    delete[] g_prof.ev;
-    delete[] g_prof.kid;
-    g_prof = Profiler();
-    return fail(MJ_GRPO_ERR_HIP, "profile set-up: %s", hipGetErrorString(e));
-  }
-  g_prof.cap = max_launches;
-  g_prof.used = 0;
-  g_prof.on = true;
+int mj_grpo_set_trace(MjGrpoTraceFn fn, void* user) {
+  g_trace.fn = fn;
+  g_trace.user = user;
   return MJ_GRPO_OK;
-}
-
-int mj_grpo_profile_end(double* total_ms, int* launches) {
-  if (!g_prof.on) return fail(MJ_GRPO_ERR_UNSUPPORTED, "profiling is not on");
-  if (!total_ms || !launches) return fail(MJ_GRPO_ERR_NULL, "total_ms/launches is NULL");
-  for (int k = 0; k < MJ_GRPO_K_COUNT; ++k) { total_ms[k] = 0.0; launches[k] = 0; }
-  int rc = MJ_GRPO_OK;
-  for (int i = 0; i < g_prof.used; ++i) {
-    float ms = 0.f;
-    hipError_t e = hipEventSynchronize(g_prof.ev[2 * i + 1]);
-    if (e == hipSuccess) e = hipEventElapsedTime(&ms, g_prof.ev[2 * i], g_prof.ev[2 * i + 1]);
-    if (e != hipSuccess) { rc = fail(MJ_GRPO_ERR_HIP, "profile event: %s", hipGetErrorString(e)); break; }
-    total_ms[g_prof.kid[i]] += ms;
-    launches[g_prof.kid[i]] += 1;
-  }
-  for (int i = 0; i < 2 * g_prof.cap; ++i) (void)hipEventDestroy(g_prof.ev[i]);
-  delete[] g_prof.ev;
-  delete[] g_prof.kid;
-  g_prof = Profiler();
-  return rc;
 }
 
 int mj_grpo_workspace_bytes(const MjGrpoDesc* desc, size_t* forward_bytes, size_t* forward_backward_bytes) {
@@ -551,6 +413,28 @@ int mj_grpo_sequence_entropy(const float* token_entropy, const float* mask, int6
   if (b <= 0 || t <= 0 || b > (1 << 24) || t > (1 << 24)) return fail(MJ_GRPO_ERR_SHAPE, "sequence_entropy: bad shape b=%lld t=%lld", (long long)b, (long long)t);
   mj::k_sequence_entropy<<<(unsigned)((b + 3) / 4), 256, 0, (hipStream_t)stream>>>(token_entropy, mask, (int)b, (int)t, entropy, entropy_loss);
   return check_launch("k_sequence_entropy");
+}
+
+int mj_grpo_scale_gradients(void* d_hidden, int64_t n, int64_t h, int64_t ld_hidden, void* d_lm_head, int64_t hw,
+                            int64_t v, int64_t ld_w, int d_lm_head_bf16, const float* scale, void* stream) {
+  if (!scale) return fail(MJ_GRPO_ERR_NULL, "scale_gradients: scale is NULL");
+  if (!d_hidden && !d_lm_head) return fail(MJ_GRPO_ERR_NULL, "scale_gradients: both gradients are NULL");
+  hipStream_t st = (hipStream_t)stream;
+  const unsigned grid = 2048;       // grid-stride: a launch whose workgroups all leave costs a few microseconds
+  if (d_hidden) {
+    if (n <= 0 || h <= 0 || ld_hidden < h || h % 8 || ld_hidden % 8)
+      return fail(MJ_GRPO_ERR_SHAPE, "scale_gradients: bad d_hidden shape n=%lld h=%lld ld=%lld", (long long)n, (long long)h, (long long)ld_hidden);
+    if (misaligned(d_hidden)) return fail(MJ_GRPO_ERR_ALIGN, "scale_gradients: d_hidden must be 16-byte aligned");
+    mj::k_scale_inplace<true><<<grid, 256, 0, st>>>(d_hidden, n, h, ld_hidden, scale);
+  }
+  if (d_lm_head) {
+    if (hw <= 0 || v <= 0 || ld_w < v || v % 8 || ld_w % 8)
+      return fail(MJ_GRPO_ERR_SHAPE, "scale_gradients: bad d_lm_head shape h=%lld v=%lld ld=%lld", (long long)hw, (long long)v, (long long)ld_w);
+    if (misaligned(d_lm_head)) return fail(MJ_GRPO_ERR_ALIGN, "scale_gradients: d_lm_head must be 16-byte aligned");
+    if (d_lm_head_bf16) mj::k_scale_inplace<true><<<grid, 256, 0, st>>>(d_lm_head, hw, v, ld_w, scale);
+    else mj::k_scale_inplace<false><<<grid, 256, 0, st>>>(d_lm_head, hw, v, ld_w, scale);
+  }
+  return check_launch("k_scale_inplace");
 }
 
 int mj_grpo_value_workspace_bytes(const MjGrpoDesc* desc, size_t* extra_bytes) {
@@ -593,24 +477,9 @@ int mj_grpo_backward(const MjGrpoDesc* desc, const void* hidden, const void* lm_
 
 }  // extern "C"
 
-// ---- measurement support
-extern "C" {
-
-int mj_grpo_probe_mfma(const void* operands, float* out, int workgroups, int iters, double* flop, void* stream) {
-  if (!operands || !out) return fail(MJ_GRPO_ERR_NULL, "probe: operands/out is NULL");
-  if (workgroups <= 0 || workgroups > (1 << 16) || iters <= 0) return fail(MJ_GRPO_ERR_SHAPE, "probe: bad workgroups/iters");
-  if (misaligned(operands)) return fail(MJ_GRPO_ERR_ALIGN, "probe: operands must be 16-byte aligned");
-  mj::k_probe_mfma<<<workgroups, 256, 0, (hipStream_t)stream>>>((const mj::bf16x8*)operands, out, iters);
-  if (flop) *flop = (double)workgroups * 4.0 * iters * 2.0 * 16.0 * 32768.0;
-  return check_launch("k_probe_mfma");
-}
-
-}  // extern "C"
-
 // ---- forward without a caller workspace: the workspace is a static device array
 namespace {
 constexpr size_t kScratchBytes = (size_t)MJ_GRPO_NOALLOC_SCRATCH_BYTES;
-constexpr int kMaxDevices = 64;
 }  // namespace
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 namespace {
@@ -642,30 +511,10 @@ int mj_grpo_forward_noalloc(const MjGrpoDesc* desc, const void* hidden, const vo
                             const float* old_logp, const float* advantages, const float* mask, float* logp,
                             float* lse, float* token_entropy, float* loss, void* stream) {
   if (desc == nullptr) return fail(MJ_GRPO_ERR_NULL, "desc is NULL");
-  MjGrpoDesc d = *desc;
+  MjGrpoDesc d;
   Plan p;
   int rc;
-  if (d.chunk_tokens > 0) {
-    if ((rc = make_plan(&d, &p))) return rc;
-  } else {
-    // the largest chunk (a multiple of 256 tokens) whose statistics fit the static array
-    int64_t lo = 1, hi = (d.n_tokens + 255) / 256;   // in units of 256 tokens
-    if (hi > 64) hi = 64;
-    d.chunk_tokens = 256;
-    if ((rc = make_plan(&d, &p))) return rc;
-    while (p.total_fwd <= kScratchBytes && lo < hi) {
-      const int64_t mid = (lo + hi + 1) / 2;
-      MjGrpoDesc t = d;
-      t.chunk_tokens = mid * 256;
-      Plan q;
-      if ((rc = make_plan(&t, &q))) return rc;
-      if (q.total_fwd <= kScratchBytes) { lo = mid; d = t; p = q; } else { hi = mid - 1; }
-    }
-  }
-  if (p.total_fwd > kScratchBytes)
-    return fail(MJ_GRPO_ERR_WORKSPACE,
-                "this shape needs %zu bytes of forward workspace with %lld-token chunks; the static array holds %zu "
-                "(use mj_grpo_forward with a caller workspace)", p.total_fwd, (long long)p.chunk, kScratchBytes);
+  if ((rc = noalloc_plan(desc, kScratchBytes, &d, &p))) return rc;
   void* ws = nullptr;
   if ((rc = scratch_address(&ws))) return rc;
   return run(kForward, &d, hidden, lm_head, targets, old_logp, advantages, mask, logp, lse, token_entropy, loss,
@@ -740,16 +589,9 @@ int mj_sample_logits(const void* hidden, int64_t ld_hidden, const void* lm_head,
   // per CU) whose items are <= 256 columns wide.  Measured at 3584 x 152064: the 128-row tile beats
   // both a 64-row tile with two workgroups per CU (0.25 against 0.23 ms at 64 rows) and, past 128
   // rows, is beaten by the 256-row tile (two 128-row tiles: 0.35 against 0.32 ms at 192 rows).
-  const int bn = b <= 128 ? 128 : 256;
-  const int64_t tiles_n = (b + bn - 1) / bn;
-  const int64_t slots = 256;
-  int64_t tile_rows = BM;
-  for (int64_t rounds = 1; rounds <= 4096; ++rounds) {
-    const int64_t per = slots * rounds / tiles_n;            // items along the vocabulary
-    if (per == 0) continue;
-    const int64_t cols = rup((vocab + per - 1) / per, 8);
-    if (cols <= BM) { tile_rows = cols; break; }
-  }
+  int bn;
+  int64_t tiles_n, tile_rows;
+  sample_tiles(b, vocab, &bn, &tiles_n, &tile_rows);
   a.tile_rows = (int)tile_rows;
   const mj::TileMap map = mj::TileMap::pick_shape((int)((vocab + tile_rows - 1) / tile_rows), (int)tiles_n, 1, 1);
   hipStream_t st = (hipStream_t)stream;

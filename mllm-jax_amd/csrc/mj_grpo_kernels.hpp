@@ -917,6 +917,33 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
   }
 }
 
+// ----------------------------------------------------------------------------- upstream gradient
+// rows x cols elements of a row-major matrix (pitch ld elements) times *scale, in place; every
+// workgroup leaves at once when *scale == 1 (the usual case: the loss is what gets differentiated).
+// BF16: 16-bit elements (8 per 16-byte unit), else float32 (4 per unit).  cols % 8 == 0.
+template <bool BF16>
+__global__ __launch_bounds__(256) void k_scale_inplace(void* data, int64_t rows, int64_t cols, int64_t ld,
+                                                       const float* scale) {
+  const float s = *scale;
+  if (s == 1.f) return;
+  constexpr int E = BF16 ? 8 : 4;
+  const int64_t per_row = cols / E, units = rows * per_row;
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += (int64_t)gridDim.x * 256) {
+    const int64_t r = u / per_row, c = (u - r * per_row) * E;
+    if (BF16) {
+      u32x4* ptr = (u32x4*)((uint16_t*)data + r * ld + c);
+      u32x4 v = *ptr;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        v[j] = pack_bf16(s * __uint_as_float(v[j] << 16), s * __uint_as_float(v[j] & 0xffff0000u));
+      *ptr = v;
+    } else {
+      f32x4* ptr = (f32x4*)((float*)data + r * ld + c);
+      *ptr = *ptr * s;
+    }
+  }
+}
+
 // ----------------------------------------------------------------------------- per-sequence entropy
 // MLLM_JAX/train_modules/__init__.py:141-157 on [b, t] row-major data, one wavefront per sequence:
 //   entropy[s]      = sum_t(H * mask) / sum_t(mask)                      (nan for an empty row, as there)

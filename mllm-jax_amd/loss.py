@@ -22,38 +22,93 @@ import torch
 
 from . import _lib
 
-_workspaces: dict[Any, torch.Tensor] = {}
+class _DeviceWorkspace:
+    """The cached workspace of one device and the stream that used it last."""
+    __slots__ = ("tensor", "stream")
+
+    def __init__(self, tensor: torch.Tensor, stream: torch.cuda.Stream):
+        self.tensor, self.stream = tensor, stream
+
+
+_workspaces: dict[Any, _DeviceWorkspace] = {}
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    # one per (device, stream): calls enqueued on different streams may overlap on the GPU and the
-    # library's rule is "two calls may overlap only if they use distinct workspaces"
-    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
+    """One workspace per device, grown on demand.  The library's rule is "two calls may overlap only
+    if they use distinct workspaces": a call on another stream than the previous one first waits for
+    everything that stream had enqueued, so calls from several streams share the buffer one after
+    the other instead of each stream keeping ~6 GB of its own.  Under stream capture the buffer is a
+    fresh allocation from the graph's own pool and is not cached: a captured address must never be
+    handed to eager code."""
+    stream = torch.cuda.current_stream(device)
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(nbytes, dtype=torch.uint8, device=device)
+    key = (device.type, device.index)
+    ent = _workspaces.get(key)
+    if ent is not None and ent.stream != stream:
+        stream.wait_event(ent.stream.record_event())
+        ent.tensor.record_stream(stream)      # the caching allocator must not recycle it under this stream
+        ent.stream = stream
+    if ent is None or ent.tensor.numel() < nbytes:
         _workspaces.pop(key, None)
-        ws = None
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+        ent = None                            # free the old buffer before asking for the larger one
+        ent = _DeviceWorkspace(torch.empty(nbytes, dtype=torch.uint8, device=device), stream)
+        _workspaces[key] = ent
+    return ent.tensor
 
 
 def release_workspaces() -> None:
-    """Drops the cached workspaces (one per device and stream)."""
+    """Drops the cached workspaces (one per device) and any cached bf16 copy of float32 weights."""
     _workspaces.clear()
+    _bf16_copies.clear()
 
 
 _bf16_copies: dict = {}      # id(tensor) -> (weak reference to it, state key, bf16 copy)
 
 
+class _Bf16Cache(threading.local):
+    depth: int = 0
+
+
+_bf16_cache = _Bf16Cache()
+
+
+@contextlib.contextmanager
+def cache_bf16_lm_head():
+    """Within this context the bf16 copy that the kernels read of a FLOAT32 lm_head is kept between
+    calls for as long as the same tensor object is unchanged (same object, same autograd version
+    counter, same storage and layout) and dropped on leaving.  The cast of [H,V] is a 3.3 GB pass at
+    the Qwen2.5-7B shape; the micro-batches and PPO epochs between two optimizer steps all read the
+    same weights (ppo_update opens this context around each of those spans).
+
+    Opt-in because the version counter does not see every write: `w.data.add_(...)`, the
+    torch._foreach_* updates of some optimizers and some checkpoint loaders change the values
+    without bumping it.  Open the context only around code that does not write the weights that
+    way, or call invalidate_bf16_lm_head() after such a write.  Outside the context every call
+    casts anew (what the reference does: param_dtype f32, dtype bf16,
+    MLLM_JAX/language/llama/llama.py:251-256)."""
+    _bf16_cache.depth += 1
+    try:
+        yield
+    finally:
+        _bf16_cache.depth -= 1
+        if _bf16_cache.depth == 0:
+            _bf16_copies.clear()
+
+
+def invalidate_bf16_lm_head() -> None:
+    """Forgets every cached bf16 copy (see cache_bf16_lm_head): call after writing float32 weights
+    through `.data` or any other route that does not bump the tensor's version counter."""
+    _bf16_copies.clear()
+
+
 def _bf16_weights(w: torch.Tensor) -> torch.Tensor:
-    """bf16 view of the lm_head for the kernels.  The reference keeps float32 master weights and
-    casts per call (param_dtype f32, dtype bf16: MLLM_JAX/language/llama/llama.py:251-256); a cast of
-    [H,V] is a 3.3 GB pass at the Qwen2.5-7B shape, so the copy is kept for as long as the same
-    tensor object has not been written to (micro-batches and PPO epochs between two optimizer
-    steps) and dropped when that tensor dies."""
+    """bf16 matrix for the kernels: the tensor itself when it is bf16, else a cast -- per call, or kept
+    under cache_bf16_lm_head()."""
     if w.dtype == torch.bfloat16:
         return w.detach()
+    if _bf16_cache.depth == 0:
+        return w.detach().to(torch.bfloat16)
     ident = id(w)                        # the caller's tensor object (detach() makes a new one per call)
     key = (w._version, w.data_ptr(), tuple(w.shape), tuple(w.stride()))
     hit = _bf16_copies.get(ident)
@@ -84,7 +139,7 @@ class _Prepared:
     def __init__(self, hidden, lm_head, target_ids, old_logps, advantages, mask, *,
                  total_valid_token_count, epsilon_low, epsilon_high, temperature,
                  final_logit_softcap, seq_shape, chunk_tokens, sft=False, accumulate=False,
-                 entropy_coef=0.0, entropy_token_count=None, skip_masked=False, dhidden_splits=0):
+                 entropy_coef=0.0, entropy_token_count=None, skip_masked=False, dhidden_splits=0, loss_scale=1.0):
         if hidden.device.type != "cuda":
             raise RuntimeError("grpo_fused_loss needs tensors on an MI355X device (got "
                                f"{hidden.device}); there is no CPU path")
@@ -134,7 +189,8 @@ class _Prepared:
         d.temperature = float(temperature)
         d.softcap = float(final_logit_softcap or 0.0)
         d.inv_total_valid_tokens = (1.0 / tv) if tv != 0 else float("inf")
-        d.grad_loss_scale = 1.0
+        self.loss_scale = float(loss_scale)
+        d.grad_loss_scale = self.loss_scale      # the kernels write gradients of loss_scale * loss
         d.dhidden_splits = int(dhidden_splits or 0)
         d.entropy_coef = float(entropy_coef)
         if entropy_coef != 0.0 or entropy_token_count is not None:
@@ -257,7 +313,7 @@ class _ValueHead:
 
 _DEFAULTS = dict(total_valid_token_count=None, epsilon_low=0.2, epsilon_high=0.3, temperature=1.0,
                  final_logit_softcap=None, seq_shape=None, chunk_tokens=None, entropy_coef=0.0,
-                 entropy_token_count=None, skip_masked=False, dhidden_splits=0)
+                 entropy_token_count=None, skip_masked=False, dhidden_splits=0, loss_scale=1.0)
 
 
 def grpo_loss_value_and_grad(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
@@ -340,15 +396,30 @@ def _poison_unless_one(grad_loss: torch.Tensor) -> torch.Tensor:
     return torch.where(g == 1, torch.zeros_like(g), torch.full_like(g, float("nan")))
 
 
+def _apply_upstream(grad_loss: torch.Tensor, d_h: torch.Tensor, d_w: Optional[torch.Tensor]) -> None:
+    """Multiplies the gradients the kernels wrote by the upstream gradient, in place and on the
+    device: when it is 1 -- the loss itself is what gets differentiated -- the launches leave at once
+    (no pass over [N,H] or [H,V], no host synchronisation)."""
+    g = grad_loss.detach().reshape(-1)[:1].to(torch.float32).contiguous()
+    with torch.cuda.device(d_h.device):
+        _lib.check(_lib.load().mj_grpo_scale_gradients(
+            d_h.data_ptr(), d_h.shape[0], d_h.shape[1], d_h.stride(0),
+            None if d_w is None else d_w.data_ptr(), 0 if d_w is None else d_w.shape[0],
+            0 if d_w is None else d_w.shape[1], 0 if d_w is None else d_w.stride(0),
+            int(d_w is not None and d_w.dtype == torch.bfloat16), g.data_ptr(),
+            torch.cuda.current_stream(d_h.device).cuda_stream))
+
+
 class _FusedLossFn(torch.autograd.Function):
-    """loss = policy loss - entropy_coef * entropy [+ value_coef * value_loss] with the gradients the
-    kernels wrote in the same pass.  value_w / value_b / value are None without a value head."""
+    """loss = loss_scale * (policy loss - entropy_coef * entropy [+ value_coef * value_loss]) with the
+    gradients the kernels wrote in the same pass.  value_w / value_b / value are None without a value
+    head.  The gradients are handed out once: a second backward through the same call raises."""
 
     @staticmethod
     def forward(ctx, hidden, lm_head, prepared: _Prepared, want_grad: bool, value_w=None, value_b=None,
                 value: Optional[_ValueHead] = None):
         ctx.direct = ctx.terminal = False
-        ctx.d_w = ctx.buf = ctx.value = None
+        ctx.d_h = ctx.d_w = ctx.buf = ctx.value = None
         if want_grad:
             # a bf16 parameter takes a bf16 gradient: the dW kernel writes it, no conversion pass
             dw_dtype = torch.bfloat16 if lm_head.dtype == torch.bfloat16 else torch.float32
@@ -356,17 +427,12 @@ class _FusedLossFn(torch.autograd.Function):
             if buf is not None:
                 _check_accumulator(buf, prepared)
                 prepared.desc.flags |= _lib.FLAG_DW_ACCUMULATE
-                d_h, _ = prepared.forward_backward(buf, value)
+                ctx.d_h, _ = prepared.forward_backward(buf, value)
                 _accumulate_target.uses += 1
                 ctx.direct, ctx.buf = True, buf
-                ctx.save_for_backward(d_h)
-            elif _accumulate_target.terminal:
-                d_h, d_w = prepared.forward_backward(None, value, dw_dtype)
-                ctx.terminal, ctx.d_w = True, d_w      # kept out of save_for_backward: poisoned in place on misuse
-                ctx.save_for_backward(d_h)
             else:
-                d_h, d_w = prepared.forward_backward(None, value, dw_dtype)
-                ctx.save_for_backward(d_h, d_w)
+                ctx.d_h, ctx.d_w = prepared.forward_backward(None, value, dw_dtype)
+                ctx.terminal = _accumulate_target.terminal
             ctx.shapes = (hidden.shape, hidden.dtype, lm_head.dtype)
             if value is not None:
                 ctx.value = (value.d_w, value.d_b, value_w.shape, value_w.dtype, value_b.shape, value_b.dtype)
@@ -375,24 +441,32 @@ class _FusedLossFn(torch.autograd.Function):
         loss = prepared.loss[0].clone()
         if value is not None and value.value_loss is not None:
             loss = loss + value.coef * value.value_loss[0]
+        if prepared.loss_scale != 1.0:
+            loss = loss * prepared.loss_scale
         return loss
 
     @staticmethod
     def backward(ctx, grad_loss):
+        if ctx.d_h is None:
+            raise RuntimeError("the fused loss hands out the gradients of a call once (they are scaled in place); "
+                               "evaluate the loss again instead of a second backward through the same call")
         shape, h_dtype, w_dtype = ctx.shapes
+        d_h, ctx.d_h = ctx.d_h, None
+        d_w, ctx.d_w = ctx.d_w, None
         if ctx.direct:
-            (d_h,) = ctx.saved_tensors
             gw = None                      # already added into the accumulator by the dW kernel ...
             ctx.buf[0, :1].add_(_poison_unless_one(grad_loss))   # ... with upstream gradient 1
+            _apply_upstream(grad_loss, d_h, None)
         elif ctx.terminal:
-            (d_h,) = ctx.saved_tensors
-            d_w, ctx.d_w = ctx.d_w, None
             d_w[0, :1].add_(_poison_unless_one(grad_loss))
-            gw = d_w if d_w.dtype == w_dtype else d_w.to(w_dtype)
+            _apply_upstream(grad_loss, d_h, None)
+            gw = d_w
         else:
-            d_h, d_w = ctx.saved_tensors
-            gw = (d_w * grad_loss).to(w_dtype)
-        gh = (d_h * grad_loss.to(d_h.dtype)).reshape(shape).to(h_dtype)
+            _apply_upstream(grad_loss, d_h, d_w)
+            gw = d_w
+        if gw is not None and gw.dtype != w_dtype:
+            gw = gw.to(w_dtype)
+        gh = d_h.reshape(shape).to(h_dtype)
         gwv = gbv = None
         if ctx.value is not None:
             d_wv, d_bv, wv_shape, wv_dtype, bv_shape, bv_dtype = ctx.value
@@ -410,7 +484,10 @@ def grpo_fused_loss(hidden, lm_head, target_ids, old_logps, advantages, mask, *,
     train_modules/__init__.py:161-165), advantages [N] (or [B] with seq_shape=(B,T)),
     mask [N] in {0,1}.  Returns {"loss", "per_token_logps", "entropy", "entropy_loss"
     [, "token_entropy"]} like train_modules/__init__.py:185-192; "loss" is differentiable
-    with respect to hidden and lm_head, everything else carries no gradient."""
+    with respect to hidden and lm_head, everything else carries no gradient.
+    `loss_scale=c` returns c * loss with the kernels writing the gradients of c * loss directly
+    (a constant known before the call, e.g. 1 / gradient-accumulation steps: multiplying the
+    returned loss afterwards gives the same result through an in-place pass over both gradients)."""
     opts = {**_DEFAULTS, **kw}
     p = _Prepared(hidden, lm_head, target_ids, old_logps, advantages, mask, **opts)
     want = torch.is_grad_enabled() and (hidden.requires_grad or lm_head.requires_grad)

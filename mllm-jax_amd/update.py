@@ -24,7 +24,7 @@ from typing import Any, Callable, Dict, Mapping, Optional
 
 import torch
 
-from .loss import accumulate_lm_head_grad_into, terminal_loss
+from .loss import accumulate_lm_head_grad_into, cache_bf16_lm_head, terminal_loss
 
 Params = Dict[str, torch.Tensor]
 
@@ -141,7 +141,7 @@ def ppo_update(*, state: Any, datas: Mapping[str, Any], total_valid_token_count:
                train_step: Callable[[Any, Any], Any] = training_step,
                slice_data: Callable[[Any, int, int], Any] = slice_data,
                grad_accum_steps: int, ppo_steps: int):
-    """update/ppo.py:6-46, kept statement for statement (a caller contract, not a redesign: the
+    """update/ppo.py:6-46, the same loop (a caller contract, not a redesign: the
     runner and the update modules call it with exactly these keywords): ppo_steps passes over the
     global batch in grad_accum_steps micro-batches.  Every micro-batch is normalised by the GLOBAL total_valid_token_count
     (:37); the first pass collects per_token_logps, which become old_per_token_logps for the
@@ -150,16 +150,19 @@ def ppo_update(*, state: Any, datas: Mapping[str, Any], total_valid_token_count:
     last_meta: Mapping[str, Any] = {}
     entropy = None
     per_token_logps = []
-    for ppo_step_idx in range(int(ppo_steps)):
-        for micro_idx in range(int(grad_accum_steps)):
-            local = {k: slice_data(v, int(grad_accum_steps), int(micro_idx)) for k, v in datas_dict.items()}
-            local["total_valid_token_count"] = total_valid_token_count
-            state, last_meta = train_step(state, local)
+    # float32 master weights are cast to bf16 once per optimizer step, not once per micro-batch: an
+    # update replaces the parameter tensors (LossTrainState.apply_gradients), which ends a cached copy
+    with cache_bf16_lm_head():
+        for ppo_step_idx in range(int(ppo_steps)):
+            for micro_idx in range(int(grad_accum_steps)):
+                local = {k: slice_data(v, int(grad_accum_steps), int(micro_idx)) for k, v in datas_dict.items()}
+                local["total_valid_token_count"] = total_valid_token_count
+                state, last_meta = train_step(state, local)
+                if ppo_step_idx == 0:
+                    per_token_logps.append(last_meta["per_token_logps"])
             if ppo_step_idx == 0:
-                per_token_logps.append(last_meta["per_token_logps"])
-        if ppo_step_idx == 0:
-            datas_dict["old_per_token_logps"] = torch.cat(per_token_logps, dim=0)
-            entropy = last_meta.get("entropy")
+                datas_dict["old_per_token_logps"] = torch.cat(per_token_logps, dim=0)
+                entropy = last_meta.get("entropy")
     return state, datas_dict, last_meta, entropy
 
 

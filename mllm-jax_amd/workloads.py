@@ -96,6 +96,20 @@ def make_workload(cfg: LossConfig, device, seed: int,
     return wl
 
 
+def gumbel_max_targets(wl: dict, gen: torch.Generator) -> torch.Tensor:
+    """`sample_fn` for make_workload: one Gumbel-max draw per token from softmax(hidden @ lm_head) at
+    temperature 1 ("targets sampled from the model's own softmax"), 1024 tokens at a time.  Input
+    generation only: plain torch on the workload's device, not the loss path."""
+    h, w = wl["hidden"].float(), wl["lm_head"].float()
+    out = torch.empty(h.shape[0], dtype=torch.int64, device=h.device)
+    g = torch.Generator(device=h.device).manual_seed(int(gen.initial_seed()) + 1)
+    for s in range(0, h.shape[0], 1024):
+        z = h[s:s + 1024] @ w
+        u = torch.rand(z.shape, generator=g, device=h.device).clamp_min(1e-20)
+        out[s:s + 1024] = (z - torch.log(-torch.log(u))).argmax(-1)
+    return out
+
+
 def flops(cfg_or_shape) -> float:
     """Algorithmic flop of one fwd+bwd: 6*N*H*V (logits, dHidden, dW)."""
     if isinstance(cfg_or_shape, LossConfig):

@@ -13,7 +13,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 @pytest.fixture(scope="module")
 def lib():
     from mllm_jax_amd import _lib, build
-    if not os.path.exists(_lib.LIB_PATH):
+    if not os.path.exists(_lib.LIB_PATH) or not os.path.exists(build.BENCH_LIB):
         build.build(verbose=False)
     return _lib
 
@@ -37,6 +37,25 @@ def test_header_symbols_are_exported(lib):
     for name in declared:
         assert hasattr(handle, name)
     assert handle.mj_grpo_version() >= 100
+
+
+def test_bench_library_exports_its_header_and_the_product_does_not(lib):
+    """Measurement support (event timing behind the launch-trace hook, the MFMA-only probe) lives in
+    libmj_grpo_bench.so / include/mj_grpo_bench.h; the product library exports none of it."""
+    header = open(os.path.join(ROOT, "include", "mj_grpo_bench.h")).read()
+    declared = set(re.findall(r"\b(mj_bench_[a-z_]+)\s*\(", header))
+    assert declared == {"mj_bench_profile_begin", "mj_bench_profile_end", "mj_bench_trace", "mj_bench_probe_mfma",
+                        "mj_bench_last_error"}
+    bench = C.CDLL(os.path.join(os.path.dirname(lib.LIB_PATH), "libmj_grpo_bench.so"))
+    product = lib.load()
+    for name in declared:
+        assert hasattr(bench, name)
+        assert not hasattr(product, name)
+    for name in ("mj_grpo_profile_begin", "mj_grpo_profile_end", "mj_grpo_probe_mfma"):
+        assert not hasattr(product, name)
+    # switching the trace hook on and off needs no device
+    assert product.mj_grpo_set_trace(C.cast(bench.mj_bench_trace, C.c_void_p), None) == 0
+    assert product.mj_grpo_set_trace(None, None) == 0
 
 
 def test_desc_layout_matches_header(lib):
@@ -175,6 +194,7 @@ def test_headers_are_plain_c_and_the_library_links_from_c(lib, tmp_path):
 #include "mj_grpo.h"
 #include "mj_norm.h"
 #include "mj_sample.h"
+#include "mj_grpo_bench.h"
 int main(void) {
   MjGrpoDesc d;
   size_t fwd = 0, both = 0;

@@ -38,16 +38,7 @@ def _make(idx, seqs=None):
                                      wl["mask"], total_valid_token_count=wl["total_valid_token_count"],
                                      **kw)["per_token_logps"]
 
-    def sample_fn(wl, gen):
-        # one Gumbel-max sample per token from softmax(h W) (targets "from the model's own softmax")
-        h, w = wl["hidden"].float(), wl["lm_head"].float()
-        out = torch.empty(h.shape[0], dtype=torch.int64, device=h.device)
-        g = torch.Generator(device=h.device).manual_seed(int(gen.initial_seed()) + 1)
-        for s in range(0, h.shape[0], 1024):
-            z = h[s:s + 1024] @ w
-            u = torch.rand(z.shape, generator=g, device=h.device).clamp_min(1e-20)
-            out[s:s + 1024] = (z - torch.log(-torch.log(u))).argmax(-1)
-        return out
+    from mllm_jax_amd.workloads import gumbel_max_targets as sample_fn
 
     wl = M.make_workload(cfg, dev, 20250 + idx, logp_fn=logp_fn, sample_fn=sample_fn, seqs=seqs)
     return M, cfg, kw, wl
