@@ -20,6 +20,7 @@
 namespace mj {
 
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f, kLn2Sq = 0.4804530139182014f;
 // Stand-in logit for vocab rows past V.  A power of two, so that kNegBig * kLog2e is exact and
 // fma(z, kLog2e, -max * kLog2e) is exactly 0 when a whole half-tile holds only stand-ins.
 constexpr float kNegBig = -0x1p100f;
@@ -178,6 +179,10 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
     // Softcap (CAP: a kernel of its own, so that the uncapped one carries none of this).  While every
     // logit of the block is small against the cap -- checked per wavefront -- tanh is its odd series
     // to u^7 (|u| <= 0.25: error below 1e-7 of u, five multiply-adds instead of an exp and a reciprocal).
+    // In kStatsExp the capped logit is kept in units of log2: t = cap(z) * log2(e), with log2(e) and the
+    // powers of 1 / cap folded into the series' coefficients, so that exp(cap(z)) = exp2(t) needs no
+    // multiply; the sums, cap'(z) and the sampled token's logit are taken from t.
+    constexpr bool kLog2Units = CAP && MODE == kStatsExp;
     if (CAP) {
       float big = 0.f;
 #pragma unroll
@@ -185,18 +190,25 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
 #pragma unroll
         for (int r = 0; r < 16; ++r) big = fmaxf(big, fabsf(g.acc[mi][ni][r]));
       if (__all(big * inv_cap <= 0.25f)) {
+        // z P(z^2),  P(w) = k (1 - w / (3 c^2) + 2 w^2 / (15 c^4) - 17 w^3 / (315 c^6)),  k = log2(e) or 1
+        const float k0 = kLog2Units ? kLog2e : 1.f;
+        const float c1 = k0 * (-1.f / 3.f) * inv_cap2, c2 = k0 * (2.f / 15.f) * inv_cap2 * inv_cap2;
+        const float c3 = k0 * (-17.f / 315.f) * inv_cap2 * inv_cap2 * inv_cap2;
 #pragma unroll
         for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float z = g.acc[mi][ni][r], u = z * inv_cap, u2 = u * u;
-            g.acc[mi][ni][r] = z * fmaf(u2, fmaf(u2, fmaf(u2, -17.f / 315.f, 2.f / 15.f), -1.f / 3.f), 1.f);
+            const float z = g.acc[mi][ni][r], w = z * z;
+            g.acc[mi][ni][r] = z * fmaf(w, fmaf(w, fmaf(w, c3, c2), c1), k0);
           }
       } else {
 #pragma unroll
         for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) g.acc[mi][ni][r] = softcap_apply(g.acc[mi][ni][r], p.cap, inv_cap);
+          for (int r = 0; r < 16; ++r) {
+            const float zc = softcap_apply(g.acc[mi][ni][r], p.cap, inv_cap);
+            g.acc[mi][ni][r] = kLog2Units ? zc * kLog2e : zc;
+          }
       }
     }
     // An opaque use of the block's 64 accumulators: with it the register allocator moves them out of
@@ -294,11 +306,11 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
             float v[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-              const float z = g.acc[mi][ni][qp * 8 + j];
-              const float e = __builtin_amdgcn_exp2f(z * kLog2e);
+              const float z = g.acc[mi][ni][qp * 8 + j];          // CAP: t = cap(z) log2(e)
+              const float e = __builtin_amdgcn_exp2f(CAP ? z : z * kLog2e);
               l += e;
               s = fmaf(e, z, s);
-              v[j] = CAP ? e * (1.f - z * z * inv_cap2) : e;
+              v[j] = CAP ? e * fmaf(z * z, -kLn2Sq * inv_cap2, 1.f) : e;   // cap' = 1 - (cap(z) / cap)^2
             }
             store_rows8<false>(v, zrs, group_off(mi, qp), (uint32_t)(mi * 32 + qp * 16) * 2);
           }
@@ -308,7 +320,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const float z = g.acc[mi][ni][r];
-            const float e = __builtin_amdgcn_exp2f(z * kLog2e);
+            const float e = __builtin_amdgcn_exp2f(CAP ? z : z * kLog2e);
             l += e;
             s = fmaf(e, z, s);
           }
@@ -318,7 +330,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
         // the entropy is that of softmax(z / T) (train_modules/__init__.py:136): its own pair of sums,
         // behind a real scalar branch so that the usual T = 1 pays nothing for it
         asm volatile("");
-        const float kt = kLog2e * p.inv_t;
+        const float kt = (CAP ? 1.f : kLog2e) * p.inv_t;
         s = 0.f;
 #pragma unroll
         for (int mi = 0; mi < G::MI; ++mi)
@@ -333,6 +345,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
       }
       l += __shfl_xor(l, 32);
       s += __shfl_xor(s, 32);
+      if (CAP) s *= kLn2;                      // sum e * cap(z) in natural units
       if (lhi == 0) {
         const int64_t o = (int64_t)(tm * 2 + wm) * p.ld_p + col;
         p.pl[o] = l;
@@ -371,7 +384,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
         for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
           for (int r = 0; r < 16; ++r) zy = (flat == mi * 16 + r) ? g.acc[mi][ni][r] : zy;
-        if (hit) p.zy[col] = zy;
+        if (hit) p.zy[col] = kLog2Units ? zy * kLn2 : zy;
       }
     }
   }
