@@ -71,7 +71,9 @@ MJ_DEV void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc07f); }
 // DEAD: the caller knows which rows (kRowK) or k-rows (kKRow) of the operand are all zero and hands
 // in a bit mask, one 64-bit word per 64 of them (bit set = zero, do not fetch).  Their loads get an
 // offset that the descriptor rejects: the registers fill with zeros and no memory request is made.
-template <int ROWS, int LAYOUT, int THREADS, bool DEAD = false>
+// FRAG: rows per MFMA fragment, 32 (v_mfma_f32_32x32x16_bf16, GemmTN) or 16 (v_mfma_f32_16x16x32_bf16,
+// GemmTN16); it selects the chunk permutation of the kRowK image.
+template <int ROWS, int LAYOUT, int THREADS, bool DEAD = false, int FRAG = 32>
 struct Operand {
   static constexpr int LD = ROWS * 8 / THREADS;
   static constexpr int RPP = THREADS / 8;          // kRowK: tile rows covered by one pass of the workgroup
@@ -88,12 +90,22 @@ struct Operand {
   int klimit;            // kRowK: chunk is inside the row iff k0 < klimit
   bool col_ok;           // kKRow: this thread's chunk lies inside the valid rows
   int rd[4];             // LDS read offsets: kRowK per k-step, kKRow per fragment
+  int rd16[2][2];        // 16-row fragments (GemmTN16), kRowK: per k-step of 32 and fragment parity
 
   // 64-byte segment permutation of the kKRow image: 8 k-rows read by one transposing read
   // ({r..r+3} and {r+8..r+11}) must land in 8 different segments of the 512-byte row.
   static MJ_DEV int sigma(int krow) { return (krow & 3) | ((krow >> 1) & 4); }
-  // 16-byte chunk permutation of the kRowK image (see the file header).
-  static MJ_DEV int swz(int r) { return (r & 7) ^ ((r >> 3) & 3); }   // depends on r mod 32 only
+  // 16-byte chunk permutation of the kRowK image (see the file header); depends on r mod 32 only.
+  // 32-row fragments (lane l reads row l % 32, chunk 2 ks + l / 32): r % 8 xor (r / 8) % 4.
+  // 16-row fragments (lane l reads row l % 16, chunk 4 ks + l / 16) conflict under that permutation
+  // (SQ_LDS_BANK_CONFLICT on every read, 3.4 ns instead of 2.6 ns per ds_read_b128 and CU).  Of the
+  // 4096 permutations that are linear in the bits of r, timed one by one on the GPU, a third are
+  // conflict free for both k-steps; this is one of them: bit 1 of r flips chunk bits 4, bit 2 flips
+  // 3, bit 3 flips 6 (bit 0 needs nothing: odd rows start in the other half of the banks).
+  static MJ_DEV int swz(int r) {
+    if (FRAG == 32) return (r & 7) ^ ((r >> 3) & 3);
+    return (((r >> 1) & 1) * 4) ^ (((r >> 2) & 1) * 3) ^ (((r >> 3) & 1) * 6);
+  }
 
   // dead: kRowK -- the words covering this tile's ROWS rows (ROWS / 64 of them);
   //       kKRow -- the words of the K extent, one per slice ((K + 63) / 64 of them).
@@ -147,6 +159,22 @@ struct Operand {
     }
   }
 
+  // Read offsets for 16-row fragments of v_mfma_f32_16x16x32_bf16: lane l supplies row l % 16,
+  // k = 8 (l / 16) + 0..7 of a 32-wide k-step.  kRowK: one 16-byte read at row (f * 16 + l % 16),
+  // chunk 4 ks + l / 16; the chunk permutation depends on the row modulo 32, i.e. on f's parity.
+  MJ_DEV void init16(int wave_row0, int t) {
+    const int lane = t & 63, l15 = lane & 15, lq = lane >> 4;
+    static_assert(LAYOUT == kRowK, "16-row fragments exist for the row-major image only");
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int par = 0; par < 2; ++par)
+        rd16[ks][par] = (wave_row0 + par * 16 + l15) * 128 + (((4 * ks + lq) ^ swz(par * 16 + l15)) << 4);
+  }
+  MJ_DEV bf16x8 frag16(const char* stage, int f, int ks) const {
+    return *(const bf16x8*)(stage + rd16[ks][f & 1] + (f >> 1) * 32 * 128);
+  }
+
   // kKRow: point the descriptor at slice `slice` (its k-rows past K fall outside and read zero).
   MJ_DEV void slice_begin(int slice) {
     if (LAYOUT == kKRow) {
@@ -171,6 +199,16 @@ struct Operand {
       *(u32x4*)(stage + st_off + i * RPP * 128) = v;
     else
       *(u32x4*)(stage + ((i & 1) ? st_off1 : st_off) + i * KPP * (ROWS * 2)) = v;
+  }
+  // one 8-byte half of chunk i (kRowK): an LDS write holds the wavefront's issue while its data
+  // leaves the registers (12 cycles per 16-byte write measured between matrix instructions, 5 per 8-byte one)
+  MJ_DEV void store_half(char* stage, int i, u32x4 v, int h) const {
+    typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+    const u32x2 w = {v[2 * h], v[2 * h + 1]};
+    if (LAYOUT == kRowK)
+      *(u32x2*)(stage + st_off + i * RPP * 128 + h * 8) = w;
+    else
+      *(u32x2*)(stage + ((i & 1) ? st_off1 : st_off) + i * KPP * (ROWS * 2) + h * 8) = w;
   }
   // MFMA fragment f (32 rows) of k-step ks.
   MJ_DEV bf16x8 frag(const char* stage, int f, int ks) const {
@@ -376,6 +414,12 @@ struct GemmTN {
       if (j < A_LD) a.store(stage, j, staged[S][j]);
       else b.store(stage + OpA::kBytes, j - A_LD, staged[S][j]);
     };
+    auto store_half = [&](auto set, int slice, int j, int h) {
+      constexpr int S = decltype(set)::value;
+      char* stage = smem + (slice & 1) * kStageBytes;
+      if (j < A_LD) a.store_half(stage, j, staged[S][j], h);
+      else b.store_half(stage + OpA::kBytes, j - A_LD, staged[S][j], h);
+    };
     bf16x8 fa[2][MI], fb[2][NI];
     auto read_one = [&](int slice, int ks, int buf, int g) {
       const char* stage = smem + (slice & 1) * kStageBytes;
@@ -439,6 +483,225 @@ struct GemmTN {
       iteration(IntTag<0>(), kt + 1);
     }
     if (kt < KT) iteration(IntTag<1>(), kt);
+  }
+};
+
+// The same 256 x 256 tile on v_mfma_f32_16x16x32_bf16, in the order that the instruction rewards.
+// A wavefront's 128 x 128 is 8 x 8 blocks of 16 x 16 and a 64-wide slice is two k-steps of 32.  The
+// two k-steps of a block are issued back to back on the same accumulator: the second instruction
+// takes the first one's result inside the matrix unit, so the accumulator is read from and written
+// to the register file once per slice instead of once per instruction.  Measured in an MFMA-only
+// loop at the socket power limit with random operands: 2146-2188 TFLOP/s in this order against
+// 1817-1874 with the accumulators in rotation (which is also held at 82 % of the issue rate by the
+// accumulator reads) and 1840 for v_mfma_f32_32x32x16_bf16 in either order.
+//
+// Blocks are walked row by row (i outer, j inner).  The B fragments of the whole slice stay in
+// registers (8 x 2 fragments); the A fragments of row i + 1 are read while row i computes (three
+// register pairs in rotation); the last two rows are walked column by column and each B fragment
+// pair is re-read for the next slice after its last use.  One barrier per slice, before those two
+// rows; the LDS writes of slice k + 1 and the global loads of slice k + 1 + DEPTH ride on rows 1..5.
+// An iteration of the loop runs from row 1 of a slice to row 0 of the next one, so that at its end
+// the youngest LDS reads are a row's time old (the compiler drains the LDS counter at a loop's top).
+//
+// The matrix instructions are written as assembly so that the result register IS the accumulator
+// operand: with all 256 accumulation registers taken the register allocator otherwise routes some
+// blocks through copies (and the wait states those need).  The first slice starts from the constant
+// 0, so nothing but these instructions ever writes an accumulator.  The compiler does not see matrix
+// instructions inside the assembly, so the wait states it would put between one of them and an
+// ordinary instruction that touches an accumulator (7 behind a four-pass instruction, 2 in front)
+// are spelled out where such an instruction can follow or precede: behind the blocks of an
+// iteration's last row (loop exit; copies on the back edge, should the allocator ever make any) and
+// in front of its first block.  They cost nothing: a block keeps the matrix unit busy for 32 cycles.
+template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK, int DEPTH = 1, bool DEAD_A = false,
+          bool DEAD_B = false>
+struct GemmTN16 {
+  static_assert(BM == 256 && BN == 256, "four wavefronts of 128 x 128");
+  static_assert(DEPTH == 1 || DEPTH == 2, "one or two slices in flight between global memory and the LDS");
+  static constexpr int kThreads = 256;
+  static constexpr int WM = 128, WN = 128;
+  static constexpr int MI = 8, NI = 8;               // 16 x 16 blocks per wavefront
+  using OpA = Operand<BM, LAY_A, kThreads, DEAD_A, 16>;
+  using OpB = Operand<BN, LAY_B, kThreads, DEAD_B, 16>;
+  static constexpr int A_LD = OpA::LD, B_LD = OpB::LD, LPS = A_LD + B_LD;
+  static constexpr int kStageBytes = OpA::kBytes + OpB::kBytes;
+  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr bool kKDead = (DEAD_A && LAY_A == kKRow) || (DEAD_B && LAY_B == kKRow);
+  static_assert(LPS <= 16, "the staged chunks of a slice ride on rows 1..5, two per five blocks");
+
+  // acc[mi][ni][r]: row = mi*16 + (lane/16)*4 + r, col = ni*16 + lane%16 within the wavefront tile
+  f32x4 acc[MI][NI];
+
+  // register pair of the A fragments of row i: rows 6 and 7 are in use together, and row 0 of the
+  // next slice is read while they are
+  static constexpr int slot(int i) { return i == 0 ? 2 : i == 5 ? 2 : (i & 1) ? 0 : 1; }
+
+  MJ_DEV void run(const __bf16* A, int rows_a, int64_t lda, const __bf16* B, int rows_b, int64_t ldb, int K,
+                  char* smem, int tid = threadIdx.x, const uint64_t* dead_a = nullptr,
+                  const uint64_t* dead_b = nullptr) {
+    const int wave = tid >> 6;
+    const int wm = wave & 1, wn = wave >> 1;
+    OpA a;
+    OpB b;
+    a.init(A, rows_a, lda, K, wm * WM, tid, dead_a);
+    b.init(B, rows_b, ldb, K, wn * WN, tid, dead_b);
+    a.init16(wm * WM, tid);
+    b.init16(wn * WN, tid);
+    KDead kd;
+    if (kKDead) kd.init(dead_a, K, tid);
+    auto slices_begin = [&](int slice) {
+      a.slice_begin(slice);
+      b.slice_begin(slice);
+      if (kKDead) kd.slice_begin(slice);
+    };
+
+    u32x4 staged[DEPTH][LPS];
+    auto load_one = [&](auto set, int slice, int j) {
+      constexpr int S = decltype(set)::value;
+      if (j < A_LD) staged[S][j] = kKDead ? a.load(slice, j, kd.lo, kd.hi) : a.load(slice, j);
+      else staged[S][j] = kKDead ? b.load(slice, j - A_LD, kd.lo, kd.hi) : b.load(slice, j - A_LD);
+    };
+    auto store_one = [&](auto set, int slice, int j) {
+      constexpr int S = decltype(set)::value;
+      char* stage = smem + (slice & 1) * kStageBytes;
+      if (j < A_LD) a.store(stage, j, staged[S][j]);
+      else b.store(stage + OpA::kBytes, j - A_LD, staged[S][j]);
+    };
+    auto store_half = [&](auto set, int slice, int j, int h) {
+      constexpr int S = decltype(set)::value;
+      char* stage = smem + (slice & 1) * kStageBytes;
+      if (j < A_LD) a.store_half(stage, j, staged[S][j], h);
+      else b.store_half(stage + OpA::kBytes, j - A_LD, staged[S][j], h);
+    };
+    bf16x8 fa[3][2], fb[NI][2];
+    auto read_a = [&](int slice, int i) {
+      const char* stage = smem + (slice & 1) * kStageBytes;
+      fa[slot(i)][0] = a.frag16(stage, i, 0);
+      fa[slot(i)][1] = a.frag16(stage, i, 1);
+    };
+    auto read_b = [&](int slice, int j) {
+      const char* stage = smem + (slice & 1) * kStageBytes + OpA::kBytes;
+      fb[j][0] = b.frag16(stage, j, 0);
+      fb[j][1] = b.frag16(stage, j, 1);
+    };
+    // first: the k-step 0..31 of block (i, j); second: its k-step 32..63, on the first one's result.
+    // A block's memory instructions sit between the two.
+    auto first = [&](auto init, auto lead, int i, int j) {
+      constexpr bool kInit = decltype(init)::value != 0, kLead = decltype(lead)::value != 0;
+      (void)fa; (void)fb; (void)acc;     // named outside the assembly too, so that the lambda captures them
+      if constexpr (kInit)
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(acc[i][j]) : "v"(fa[slot(i)][0]), "v"(fb[j][0]));
+      else if constexpr (kLead)
+        asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fa[slot(i)][0]), "v"(fb[j][0]));
+      else
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fa[slot(i)][0]), "v"(fb[j][0]));
+    };
+    auto second = [&](auto settle, int i, int j) {
+      constexpr bool kSettle = decltype(settle)::value != 0;
+      (void)fa; (void)fb; (void)acc;
+      if constexpr (kSettle)
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\ts_nop 9" : "+a"(acc[i][j]) : "v"(fa[slot(i)][1]), "v"(fb[j][1]));
+      else
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fa[slot(i)][1]), "v"(fb[j][1]));
+    };
+
+    const int KT = (K + kBK - 1) / kBK;
+    slices_begin(0);
+#pragma unroll
+    for (int j = 0; j < LPS; ++j) load_one(IntTag<0>(), 0, j);
+    slices_begin(1);
+    if (DEPTH == 2) {
+#pragma unroll
+      for (int j = 0; j < LPS; ++j) load_one(IntTag<DEPTH - 1>(), 1, j);
+      slices_begin(2);
+    }
+#pragma unroll
+    for (int j = 0; j < LPS; ++j) {
+      store_one(IntTag<0>(), 0, j);
+      load_one(IntTag<0>(), DEPTH, j);
+    }
+    wait_lgkmcnt0();
+    __builtin_amdgcn_s_barrier();       // slice 0 is in LDS, the next DEPTH slices are on their way to the registers
+    read_a(0, 0);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) read_b(0, j);
+
+    auto mem_op = [&](auto set, int kt, int q) {
+      if (q < 0) return;
+      if (q / 5 >= LPS) return;
+      if (q % 5 == 0) store_half(set, kt + 1, q / 5, 0);
+      if (q % 5 == 2) store_half(set, kt + 1, q / 5, 1);
+      if (q % 5 == 4) load_one(set, kt + 1 + DEPTH, q / 5);
+    };
+    // Row i < 6 of slice kt.  set: the staging registers that hold slice kt+1 (refilled with slice
+    // kt+1+DEPTH).
+    auto row = [&](auto init, auto settle, auto set, int kt, int i) {
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        const int g = (i - 1) * NI + j;
+        if (i == 1 && j == 0) first(init, IntTag<1>(), i, j);
+        else first(init, IntTag<0>(), i, j);
+        __builtin_amdgcn_sched_barrier(0);
+        if (j == 0) read_a(kt, i + 1);
+        if (i == 5 && j == 1) read_a(kt, 7);
+        if (i == 0 && j == 1 && kt > 0) read_b(kt, NI - 1);   // the last B pair, left over by rows_back
+        // Rows 1..5 have 80 gaps (one inside each block, one behind it); chunk c takes gaps 5c, 5c+2
+        // and 5c+4: its two 8-byte halves go to the LDS, then its register is refilled (a load issued
+        // right behind the LDS write of the same registers waits until the LDS has taken them).
+        mem_op(set, kt, i == 0 ? -1 : 2 * g);
+        __builtin_amdgcn_sched_barrier(0);
+        if (j == NI - 1) second(settle, i, j);
+        else second(IntTag<0>(), i, j);
+        __builtin_amdgcn_sched_barrier(0);
+        if (i > 0 && ((2 * g + 1) % 5 == 0 || (2 * g + 1) % 5 == 2 || (2 * g + 1) % 5 == 4)) {
+          mem_op(set, kt, 2 * g + 1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    };
+    // Rows 6 and 7 of slice kt, column by column, so that the B pairs are released one per two blocks:
+    // each is re-read for slice kt+1 after its last use (inside the next column's first block; the
+    // last one inside row 0), behind the barrier that publishes that slice in the LDS.
+    auto rows_back = [&](auto init, int kt) {
+      wait_lgkmcnt0();                  // own reads of slice kt and writes of slice kt+1 are done
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        first(init, IntTag<0>(), MI - 2, j);
+        __builtin_amdgcn_sched_barrier(0);
+        if (j == 0) read_a(kt + 1, 0);
+        if (j > 0) read_b(kt + 1, j - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        second(IntTag<0>(), MI - 2, j);
+        __builtin_amdgcn_sched_barrier(0);
+        first(init, IntTag<0>(), MI - 1, j);
+        __builtin_amdgcn_sched_barrier(0);
+        second(IntTag<0>(), MI - 1, j);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // The last iteration's row 0 multiplies the zero-filled stage of a slice past K.
+    auto iteration = [&](auto init, auto set, int kt) {
+      slices_begin(kt + 1 + DEPTH);
+#pragma unroll
+      for (int i = 1; i < MI - 2; ++i) row(init, IntTag<0>(), set, kt, i);
+      rows_back(init, kt);
+      row(IntTag<0>(), IntTag<1>(), set, kt + 1, 0);
+    };
+    row(IntTag<1>(), IntTag<0>(), IntTag<0>(), 0, 0);
+    if (DEPTH == 1) {
+      iteration(IntTag<1>(), IntTag<0>(), 0);
+      for (int kt = 1; kt < KT; ++kt) iteration(IntTag<0>(), IntTag<0>(), kt);
+    } else {
+      // slice kt+1 waits in set (kt+1) % 2; unrolled by two so that the set is a compile-time constant
+      iteration(IntTag<1>(), IntTag<DEPTH - 1>(), 0);
+      int kt = 1;
+      for (; kt + 1 < KT; kt += 2) {
+        iteration(IntTag<0>(), IntTag<0>(), kt);
+        iteration(IntTag<0>(), IntTag<DEPTH - 1>(), kt + 1);
+      }
+      if (kt < KT) iteration(IntTag<0>(), IntTag<0>(), kt);
+    }
   }
 };
 

@@ -732,10 +732,8 @@ struct DhArgs {
 
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
-  using G = GemmTN<BM, BN, kRowK, kRowK, 1, true, false>;   // rows of dead tokens are not fetched
+  using G = GemmTN16<BM, BN, kRowK, kRowK, 1, true, false>;   // rows of dead tokens are not fetched
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  // Only token tiles that hold live tokens are walked: the tile list is rebuilt for that many
-  // rows of tiles, so that the live work spreads evenly over the XCDs (ids past its end leave).
   const TileMap live(live_pad(p.n_live, p.c0, p.n_pad) / BM, map.tiles_n, map.n_first, map.lgm, map.splits, map.lgs);
   int tm, tn, split;
   if (!live.tile(blockIdx.x, tm, tn, split)) return;
@@ -746,48 +744,43 @@ __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
   g.run(p.dzt + (int64_t)m0 * p.ld_z + k0, p.n - m0, p.ld_z, p.w + (int64_t)n0 * p.ld_w + k0, p.H - n0, p.ld_w,
         klen, smem, threadIdx.x, p.dead + m0 / 64);
   const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps descriptors in SGPRs
-  const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
-  const int row0 = m0 + wm * G::WM;                       // first token row of this wavefront
-  const int rows = min(max(p.n - row0, 0), G::WM);        // rows at or past n are dropped
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave & 1, wn = wave >> 1, l15 = lane & 15, lq = lane >> 4;
+  const int row0 = m0 + wm * G::WM;
+  const int rows = min(max(p.n - row0, 0), G::WM);
   if (p.splits == 1) {
     const bool scaled = __builtin_amdgcn_readfirstlane(*p.state) == 0;
     const uint32_t ld2 = (uint32_t)p.ld_dh * 2;
     const __amdgpu_buffer_rsrc_t rs = make_rsrc_wave(p.dh + (int64_t)row0 * p.ld_dh, (int64_t)rows * ld2);
-    const __amdgpu_buffer_rsrc_t srs = make_rsrc_wave(p.rs + row0, (int64_t)rows * 4);   // rows past n read 0
+    const __amdgpu_buffer_rsrc_t srs = make_rsrc_wave(p.rs + row0, (int64_t)rows * 4);
     const __amdgpu_buffer_rsrc_t dvs = make_rsrc_wave(p.dv == nullptr ? nullptr : p.dv + row0, (int64_t)rows * 4);
 #pragma unroll
-    for (int mi = 0; mi < G::MI; ++mi)
+    for (int mi = 0; mi < G::MI; ++mi) {
+      f32x4 sc = {1.f, 1.f, 1.f, 1.f}, dvr = {0.f, 0.f, 0.f, 0.f};
+      if (scaled) sc = load_b128(srs, (uint32_t)(lq * 16), (uint32_t)(mi * 16) * 4);
+      if (p.dv != nullptr) dvr = load_b128(dvs, (uint32_t)(lq * 16), (uint32_t)(mi * 16) * 4);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        // the four consecutive token rows of this lane in the 8-row group q of block mi
-        f32x4 sc = {1.f, 1.f, 1.f, 1.f}, dvr = {0.f, 0.f, 0.f, 0.f};
-        if (scaled) sc = load_b128(srs, (uint32_t)(lhi * 16), (uint32_t)(mi * 32 + q * 8) * 4);
-        if (p.dv != nullptr) dvr = load_b128(dvs, (uint32_t)(lhi * 16), (uint32_t)(mi * 32 + q * 8) * 4);
+      for (int ni = 0; ni < G::NI; ++ni) {
+        const int col = n0 + wn * G::WN + ni * 16 + l15;
+        const uint32_t voff = col < p.H ? (uint32_t)(lq * 4 * ld2 + col * 2) : kOob;
+        const float wvc = (p.dv != nullptr && col < p.H) ? p.wv[col] : 0.f;
 #pragma unroll
-        for (int ni = 0; ni < G::NI; ++ni) {
-          const int col = n0 + wn * G::WN + ni * 32 + l31;
-          const uint32_t voff = col < p.H ? (uint32_t)(lhi * 4 * ld2 + col * 2) : kOob;
-          const float wvc = (p.dv != nullptr && col < p.H) ? p.wv[col] : 0.f;
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            store_b16(f32_to_bf16(fmaf(dvr[j], wvc, g.acc[mi][ni][q * 4 + j] * sc[j])), rs, voff,
-                      (uint32_t)(mi * 32 + q * 8 + j) * ld2);
-        }
+        for (int j = 0; j < 4; ++j)
+          store_b16(f32_to_bf16(fmaf(dvr[j], wvc, g.acc[mi][ni][j] * sc[j])), rs, voff, (uint32_t)(mi * 16 + j) * ld2);
       }
+    }
   } else {
     const uint32_t ld4 = (uint32_t)p.H * 4;
     const __amdgpu_buffer_rsrc_t rs =
         make_rsrc_wave(p.part + ((int64_t)split * p.n_pad + row0) * p.H, (int64_t)rows * ld4);
 #pragma unroll
     for (int ni = 0; ni < G::NI; ++ni) {
-      const int col = n0 + wn * G::WN + ni * 32 + l31;
-      const uint32_t voff = col < p.H ? (uint32_t)(lhi * 4 * ld4 + col * 4) : kOob;
+      const int col = n0 + wn * G::WN + ni * 16 + l15;
+      const uint32_t voff = col < p.H ? (uint32_t)(lq * 4 * ld4 + col * 4) : kOob;
 #pragma unroll
       for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          store_b32(g.acc[mi][ni][r], rs, voff, (uint32_t)(mi * 32 + (r >> 2) * 8 + (r & 3)) * ld4);
+        for (int r = 0; r < 4; ++r) store_b32(g.acc[mi][ni][r], rs, voff, (uint32_t)(mi * 16 + r) * ld4);
     }
   }
 }
