@@ -90,11 +90,20 @@ struct Operand {
   int klimit;            // kRowK: chunk is inside the row iff k0 < klimit
   bool col_ok;           // kKRow: this thread's chunk lies inside the valid rows
   int rd[4];             // LDS read offsets: kRowK per k-step, kKRow per fragment
-  int rd16[2][2];        // 16-row fragments (GemmTN16), kRowK: per k-step of 32 and fragment parity
+  int rd16[LAYOUT == kRowK ? 4 : 8];   // 16-row fragments (GemmTN16): kRowK per (k-step of 32, fragment parity), kKRow per fragment
 
   // 64-byte segment permutation of the kKRow image: 8 k-rows read by one transposing read
   // ({r..r+3} and {r+8..r+11}) must land in 8 different segments of the 512-byte row.
   static MJ_DEV int sigma(int krow) { return (krow & 3) | ((krow >> 1) & 4); }
+  // The k-major image for 16-row fragments.  One transposing read fetches, per 16-lane group g, the 32
+  // bytes of the fragment's rows from the k-rows 8 g + 0..3: 16 k-rows at the same place of their 512
+  // bytes, which all start in the same bank.  perm16 moves the 32-byte pairs of 16-byte chunks of a
+  // k-row around (xor on chunk bits 1..4, a function of k-row bits 0, 1 and 3) so that the 16 pieces
+  // of one read fall into different banks; found by timing all 65536 maps that are linear in k-row
+  // bits 0, 1, 3, 4 on the GPU (a third of them are conflict free; the segment permutation above
+  // costs 2.5 ns instead of 1.9 ns per read and CU with this access pattern).
+  static MJ_DEV int perm16(int krow) { return ((krow & 1) * 12) ^ (((krow >> 1) & 1) * 6) ^ (((krow >> 3) & 1) * 5); }
+  static MJ_DEV int kperm(int krow) { return FRAG == 16 ? (perm16(krow) << 1) : (sigma(krow) << 2); }
   // 16-byte chunk permutation of the kRowK image (see the file header); depends on r mod 32 only.
   // 32-row fragments (lane l reads row l % 32, chunk 2 ks + l / 32): r % 8 xor (r / 8) % 4.
   // 16-row fragments (lane l reads row l % 16, chunk 4 ks + l / 16) conflict under that permutation
@@ -144,8 +153,8 @@ struct Operand {
       for (int i = 0; i < LD; ++i) goff[i] = (uint32_t)((krow + KPP * i) * ld2 + chunk * 16);
       col_ok = chunk * 8 < rows;
       klimit = 0;
-      st_off = krow * (ROWS * 2) + ((chunk ^ (sigma(krow) << 2)) << 4);
-      st_off1 = krow * (ROWS * 2) + ((chunk ^ (sigma(krow + KPP) << 2)) << 4);   // differs only if KPP == 8
+      st_off = krow * (ROWS * 2) + ((chunk ^ kperm(krow)) << 4);
+      st_off1 = krow * (ROWS * 2) + ((chunk ^ kperm(krow + KPP)) << 4);   // differs only if KPP == 8
       // Transposing read: the 16 lanes of a group fetch 4 k-rows x 4 row-quads (8 bytes each) and
       // get back, lane i, the 4 k of row i.  Lane l: group g = l/16, s = l%16 reads k-row
       // (g/2)*8 + s/4 (+4 for the second read, +16*ks), quad (g%2)*4 + s%4 of the 32-row fragment.
@@ -162,17 +171,34 @@ struct Operand {
   // Read offsets for 16-row fragments of v_mfma_f32_16x16x32_bf16: lane l supplies row l % 16,
   // k = 8 (l / 16) + 0..7 of a 32-wide k-step.  kRowK: one 16-byte read at row (f * 16 + l % 16),
   // chunk 4 ks + l / 16; the chunk permutation depends on the row modulo 32, i.e. on f's parity.
+  // kKRow: two transposing reads; lane l = 16 g + s addresses k-row 8 g + s / 4 (+ 4 for the second
+  // read, + 32 ks), quad s % 4 of the fragment's four, and gets back the four k of row s.
   MJ_DEV void init16(int wave_row0, int t) {
+    static_assert(FRAG == 16, "16-row fragments: the operand's image must be laid out for them");
     const int lane = t & 63, l15 = lane & 15, lq = lane >> 4;
-    static_assert(LAYOUT == kRowK, "16-row fragments exist for the row-major image only");
+    if (LAYOUT == kRowK) {
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
+      for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-      for (int par = 0; par < 2; ++par)
-        rd16[ks][par] = (wave_row0 + par * 16 + l15) * 128 + (((4 * ks + lq) ^ swz(par * 16 + l15)) << 4);
+        for (int par = 0; par < 2; ++par)
+          rd16[ks * 2 + par] = (wave_row0 + par * 16 + l15) * 128 + (((4 * ks + lq) ^ swz(par * 16 + l15)) << 4);
+    } else {
+      const int kr = 8 * lq + (l15 >> 2);
+#pragma unroll
+      for (int f = 0; f < 8; ++f) {
+        const int quad = (wave_row0 + f * 16) / 4 + (l15 & 3);
+        rd16[f] = kr * (ROWS * 2) + (((quad >> 1) ^ kperm(kr)) << 4) + (quad & 1) * 8;
+      }
+    }
   }
   MJ_DEV bf16x8 frag16(const char* stage, int f, int ks) const {
-    return *(const bf16x8*)(stage + rd16[ks][f & 1] + (f >> 1) * 32 * 128);
+    if (LAYOUT == kRowK) return *(const bf16x8*)(stage + rd16[ks * 2 + (f & 1)] + (f >> 1) * 32 * 128);
+    typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+    const char* p = stage + rd16[f] + ks * 32 * (ROWS * 2);
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * (ROWS * 2)));
+    const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, v);
   }
 
   // kKRow: point the descriptor at slice `slice` (its k-rows past K fall outside and read zero).
@@ -512,11 +538,11 @@ struct GemmTN {
 // are spelled out where such an instruction can follow or precede: behind the blocks of an
 // iteration's last row (loop exit; copies on the back edge, should the allocator ever make any) and
 // in front of its first block.  They cost nothing: a block keeps the matrix unit busy for 32 cycles.
-template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK, int DEPTH = 1, bool DEAD_A = false,
-          bool DEAD_B = false>
+template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK, bool DEAD_A = false, bool DEAD_B = false>
 struct GemmTN16 {
   static_assert(BM == 256 && BN == 256, "four wavefronts of 128 x 128");
-  static_assert(DEPTH == 1 || DEPTH == 2, "one or two slices in flight between global memory and the LDS");
+  static constexpr int DEPTH = 1;   // slices in flight between global memory and the LDS (a second set of
+                                    // staging registers, two slices in flight, measured no faster here)
   static constexpr int kThreads = 256;
   static constexpr int WM = 128, WN = 128;
   static constexpr int MI = 8, NI = 8;               // 16 x 16 blocks per wavefront
@@ -525,7 +551,7 @@ struct GemmTN16 {
   static constexpr int A_LD = OpA::LD, B_LD = OpB::LD, LPS = A_LD + B_LD;
   static constexpr int kStageBytes = OpA::kBytes + OpB::kBytes;
   static constexpr int kLdsBytes = 2 * kStageBytes;
-  static constexpr bool kKDead = (DEAD_A && LAY_A == kKRow) || (DEAD_B && LAY_B == kKRow);
+  static_assert(!(DEAD_A && LAY_A == kKRow) && !(DEAD_B && LAY_B == kKRow), "row masks only (row-major operands)");
   static_assert(LPS <= 16, "the staged chunks of a slice ride on rows 1..5, two per five blocks");
 
   // acc[mi][ni][r]: row = mi*16 + (lane/16)*4 + r, col = ni*16 + lane%16 within the wavefront tile
@@ -546,19 +572,16 @@ struct GemmTN16 {
     b.init(B, rows_b, ldb, K, wn * WN, tid, dead_b);
     a.init16(wm * WM, tid);
     b.init16(wn * WN, tid);
-    KDead kd;
-    if (kKDead) kd.init(dead_a, K, tid);
     auto slices_begin = [&](int slice) {
       a.slice_begin(slice);
       b.slice_begin(slice);
-      if (kKDead) kd.slice_begin(slice);
     };
 
     u32x4 staged[DEPTH][LPS];
     auto load_one = [&](auto set, int slice, int j) {
       constexpr int S = decltype(set)::value;
-      if (j < A_LD) staged[S][j] = kKDead ? a.load(slice, j, kd.lo, kd.hi) : a.load(slice, j);
-      else staged[S][j] = kKDead ? b.load(slice, j - A_LD, kd.lo, kd.hi) : b.load(slice, j - A_LD);
+      if (j < A_LD) staged[S][j] = a.load(slice, j);
+      else staged[S][j] = b.load(slice, j - A_LD);
     };
     auto store_one = [&](auto set, int slice, int j) {
       constexpr int S = decltype(set)::value;
@@ -573,10 +596,13 @@ struct GemmTN16 {
       else b.store_half(stage + OpA::kBytes, j - A_LD, staged[S][j], h);
     };
     bf16x8 fa[3][2], fb[NI][2];
-    auto read_a = [&](int slice, int i) {
+    auto read_a_half = [&](int slice, int i, int ks) {
       const char* stage = smem + (slice & 1) * kStageBytes;
-      fa[slot(i)][0] = a.frag16(stage, i, 0);
-      fa[slot(i)][1] = a.frag16(stage, i, 1);
+      fa[slot(i)][ks] = a.frag16(stage, i, ks);
+    };
+    auto read_a = [&](int slice, int i) {
+      read_a_half(slice, i, 0);
+      read_a_half(slice, i, 1);
     };
     auto read_b = [&](int slice, int j) {
       const char* stage = smem + (slice & 1) * kStageBytes + OpA::kBytes;
@@ -609,11 +635,6 @@ struct GemmTN16 {
 #pragma unroll
     for (int j = 0; j < LPS; ++j) load_one(IntTag<0>(), 0, j);
     slices_begin(1);
-    if (DEPTH == 2) {
-#pragma unroll
-      for (int j = 0; j < LPS; ++j) load_one(IntTag<DEPTH - 1>(), 1, j);
-      slices_begin(2);
-    }
 #pragma unroll
     for (int j = 0; j < LPS; ++j) {
       store_one(IntTag<0>(), 0, j);
@@ -641,9 +662,10 @@ struct GemmTN16 {
         if (i == 1 && j == 0) first(init, IntTag<1>(), i, j);
         else first(init, IntTag<0>(), i, j);
         __builtin_amdgcn_sched_barrier(0);
-        if (j == 0) read_a(kt, i + 1);
-        if (i == 5 && j == 1) read_a(kt, 7);
-        if (i == 0 && j == 1 && kt > 0) read_b(kt, NI - 1);   // the last B pair, left over by rows_back
+        // the A pair of the next row, one fragment per block (row 5: of the next two rows)
+        if (j < 2) read_a_half(kt, i + 1, j);
+        if (i == 5 && (j == 2 || j == 3)) read_a_half(kt, 7, j - 2);
+        if (i == 0 && j == 2 && kt > 0) read_b(kt, NI - 1);   // the last B pair, left over by rows_back
         // Rows 1..5 have 80 gaps (one inside each block, one behind it); chunk c takes gaps 5c, 5c+2
         // and 5c+4: its two 8-byte halves go to the LDS, then its register is refilled (a load issued
         // right behind the LDS write of the same registers waits until the LDS has taken them).
@@ -669,7 +691,7 @@ struct GemmTN16 {
       for (int j = 0; j < NI; ++j) {
         first(init, IntTag<0>(), MI - 2, j);
         __builtin_amdgcn_sched_barrier(0);
-        if (j == 0) read_a(kt + 1, 0);
+        if (j < 2) read_a_half(kt + 1, 0, j);
         if (j > 0) read_b(kt + 1, j - 1);
         __builtin_amdgcn_sched_barrier(0);
         second(IntTag<0>(), MI - 2, j);
@@ -689,19 +711,8 @@ struct GemmTN16 {
       row(IntTag<0>(), IntTag<1>(), set, kt + 1, 0);
     };
     row(IntTag<1>(), IntTag<0>(), IntTag<0>(), 0, 0);
-    if (DEPTH == 1) {
-      iteration(IntTag<1>(), IntTag<0>(), 0);
-      for (int kt = 1; kt < KT; ++kt) iteration(IntTag<0>(), IntTag<0>(), kt);
-    } else {
-      // slice kt+1 waits in set (kt+1) % 2; unrolled by two so that the set is a compile-time constant
-      iteration(IntTag<1>(), IntTag<DEPTH - 1>(), 0);
-      int kt = 1;
-      for (; kt + 1 < KT; kt += 2) {
-        iteration(IntTag<0>(), IntTag<0>(), kt);
-        iteration(IntTag<0>(), IntTag<DEPTH - 1>(), kt + 1);
-      }
-      if (kt < KT) iteration(IntTag<0>(), IntTag<0>(), kt);
-    }
+    iteration(IntTag<1>(), IntTag<0>(), 0);
+    for (int kt = 1; kt < KT; ++kt) iteration(IntTag<0>(), IntTag<0>(), kt);
   }
 };
 

@@ -150,7 +150,8 @@ MJ_DEV void store_rows8(const float (&v)[8], __amdgpu_buffer_rsrc_t rs, uint32_t
   __builtin_amdgcn_raw_buffer_store_b128(out, rs, voff, soff, 0);
 }
 
-// One 256 x 256 tile: logits^T [vocab x tokens] = W^T * hidden^T on MFMA, then the epilogue of MODE.
+// One 256 x 256 tile: logits^T [vocab x tokens] = W^T * hidden^T on MFMA, then the epilogue of MODE
+// (kStatsMax, kStatsGrad; kStatsExp has a tile of its own, logits_tile16).
 template <int BM, int BN, int MODE, bool CAP>
 MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid) {
   using G = GemmTN<BM, BN, kKRow, kRowK>;
@@ -179,10 +180,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
     // Softcap (CAP: a kernel of its own, so that the uncapped one carries none of this).  While every
     // logit of the block is small against the cap -- checked per wavefront -- tanh is its odd series
     // to u^7 (|u| <= 0.25: error below 1e-7 of u, five multiply-adds instead of an exp and a reciprocal).
-    // In kStatsExp the capped logit is kept in units of log2: t = cap(z) * log2(e), with log2(e) and the
-    // powers of 1 / cap folded into the series' coefficients, so that exp(cap(z)) = exp2(t) needs no
-    // multiply; the sums, cap'(z) and the sampled token's logit are taken from t.
-    constexpr bool kLog2Units = CAP && MODE == kStatsExp;
+    static_assert(MODE != kStatsExp, "kStatsExp runs on logits_tile16");
     if (CAP) {
       float big = 0.f;
 #pragma unroll
@@ -191,7 +189,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
         for (int r = 0; r < 16; ++r) big = fmaxf(big, fabsf(g.acc[mi][ni][r]));
       if (__all(big * inv_cap <= 0.25f)) {
         // z P(z^2),  P(w) = k (1 - w / (3 c^2) + 2 w^2 / (15 c^4) - 17 w^3 / (315 c^6)),  k = log2(e) or 1
-        const float k0 = kLog2Units ? kLog2e : 1.f;
+        const float k0 = 1.f;
         const float c1 = k0 * (-1.f / 3.f) * inv_cap2, c2 = k0 * (2.f / 15.f) * inv_cap2 * inv_cap2;
         const float c3 = k0 * (-17.f / 315.f) * inv_cap2 * inv_cap2 * inv_cap2;
 #pragma unroll
@@ -207,7 +205,7 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const float zc = softcap_apply(g.acc[mi][ni][r], p.cap, inv_cap);
-            g.acc[mi][ni][r] = kLog2Units ? zc * kLog2e : zc;
+            g.acc[mi][ni][r] = zc;
           }
       }
     }
@@ -296,62 +294,6 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
             store_rows8<true>(v, zrs, group_off(mi, qp), (uint32_t)(mi * 32 + qp * 16) * 2);
           }
       }
-    } else if (MODE == kStatsExp) {
-      float l = 0.f, s = 0.f;
-      if (store) {
-#pragma unroll
-        for (int mi = 0; mi < G::MI; ++mi)
-#pragma unroll
-          for (int qp = 0; qp < 2; ++qp) {
-            float v[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              const float z = g.acc[mi][ni][qp * 8 + j];          // CAP: t = cap(z) log2(e)
-              const float e = __builtin_amdgcn_exp2f(CAP ? z : z * kLog2e);
-              l += e;
-              s = fmaf(e, z, s);
-              v[j] = CAP ? e * fmaf(z * z, -kLn2Sq * inv_cap2, 1.f) : e;   // cap' = 1 - (cap(z) / cap)^2
-            }
-            store_rows8<false>(v, zrs, group_off(mi, qp), (uint32_t)(mi * 32 + qp * 16) * 2);
-          }
-      } else {
-#pragma unroll
-        for (int mi = 0; mi < G::MI; ++mi)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float z = g.acc[mi][ni][r];
-            const float e = __builtin_amdgcn_exp2f(CAP ? z : z * kLog2e);
-            l += e;
-            s = fmaf(e, z, s);
-          }
-      }
-      float lt = 0.f;
-      if (p.inv_t != 1.f) {
-        // the entropy is that of softmax(z / T) (train_modules/__init__.py:136): its own pair of sums,
-        // behind a real scalar branch so that the usual T = 1 pays nothing for it
-        asm volatile("");
-        const float kt = (CAP ? 1.f : kLog2e) * p.inv_t;
-        s = 0.f;
-#pragma unroll
-        for (int mi = 0; mi < G::MI; ++mi)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float z = g.acc[mi][ni][r];
-            const float e = __builtin_amdgcn_exp2f(z * kt);
-            lt += e;
-            s = fmaf(e, z, s);
-          }
-        lt += __shfl_xor(lt, 32);
-      }
-      l += __shfl_xor(l, 32);
-      s += __shfl_xor(s, 32);
-      if (CAP) s *= kLn2;                      // sum e * cap(z) in natural units
-      if (lhi == 0) {
-        const int64_t o = (int64_t)(tm * 2 + wm) * p.ld_p + col;
-        p.pl[o] = l;
-        p.ps[o] = s;
-        if (p.inv_t != 1.f) p.plt[o] = lt;
-      }
     } else {   // kStatsGrad
       const float lse2 = col < p.n ? p.lse[col] * kLog2e : 0.f;
       const float gneg = col < p.n ? -p.g[col] : 0.f;
@@ -384,7 +326,165 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
         for (int mi = 0; mi < G::MI; ++mi)
 #pragma unroll
           for (int r = 0; r < 16; ++r) zy = (flat == mi * 16 + r) ? g.acc[mi][ni][r] : zy;
-        if (hit) p.zy[col] = kLog2Units ? zy * kLn2 : zy;
+        if (hit) p.zy[col] = zy;
+      }
+    }
+  }
+}
+
+// The kStatsExp tile on the chained 16 x 16 x 32 engine (GemmTN16).  A lane holds, for the token
+// ni*16 + lane%16, the four vocab rows mi*16 + (lane/16)*4 + 0..3 of each of the eight blocks mi.
+// Two blocks at a time, the lanes l and l + 16 exchange one packed half (v_permlane16_swap) so that
+// each owns eight CONSECUTIVE vocab entries of one block and stores them with one 16-byte access.
+template <int BM, int BN, bool CAP>
+MJ_DEV void logits_tile16(const LogitsArgs& p, int tm, int tn, char* smem, int tid) {
+  using G = GemmTN16<BM, BN, kKRow, kRowK>;
+  const int m0 = tm * BM, n0 = tn * BN;
+  G g;
+  g.run(p.w + m0, p.V - m0, p.ld_w, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0, p.ld_hid, p.H, smem, tid);
+
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps descriptors in SGPRs
+  const int wm = wave & 1, wn = wave >> 1, l15 = lane & 15, lq = lane >> 4;
+  const int vwave = m0 + wm * G::WM;             // first vocab row of this wavefront
+  const int vbase = vwave + lq * 4;              // + mi*16 + r
+  const int t0 = n0 + wn * G::WN;                // first token of this wavefront
+  const bool tail = (m0 + BM > p.V);
+  const float inv_cap = CAP ? 1.f / p.cap : 0.f;
+  const float inv_cap2 = inv_cap * inv_cap;
+  const int zt_cols = live_pad(p.n_live, p.c0, (p.n + 255) & ~255);
+  const uint32_t ldz2 = (uint32_t)p.ld_z * 2;
+  const int trows = min(max(p.n - t0, 0), G::WN);
+  const __amdgpu_buffer_rsrc_t zrs =
+      make_rsrc_wave(p.zt == nullptr ? nullptr : p.zt + (int64_t)t0 * p.ld_z, (int64_t)trows * ldz2);
+#pragma unroll
+  for (int ni = 0; ni < G::NI; ++ni) {
+    const int col = t0 + ni * 16 + l15;
+    // softcap: see logits_tile (series while every logit of the wavefront's block column is small
+    // against the cap; the capped logit is kept in units of log2)
+    if (CAP) {
+      float big = 0.f;
+#pragma unroll
+      for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) big = fmaxf(big, fabsf(g.acc[mi][ni][r]));
+      if (__all(big * inv_cap <= 0.25f)) {
+        const float c1 = kLog2e * (-1.f / 3.f) * inv_cap2, c2 = kLog2e * (2.f / 15.f) * inv_cap2 * inv_cap2;
+        const float c3 = kLog2e * (-17.f / 315.f) * inv_cap2 * inv_cap2 * inv_cap2;
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float z = g.acc[mi][ni][r], w = z * z;
+            g.acc[mi][ni][r] = z * fmaf(w, fmaf(w, fmaf(w, c3, c2), c1), kLog2e);
+          }
+      } else {
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) g.acc[mi][ni][r] = softcap_apply(g.acc[mi][ni][r], p.cap, inv_cap) * kLog2e;
+      }
+    }
+    // an opaque use of the column's 32 accumulators: the register allocator then moves them out of the
+    // accumulation registers here, one column at a time, instead of parking some in scratch memory
+#pragma unroll
+    for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(g.acc[mi][ni][r]));
+    if (tail) {
+      asm volatile("");
+#pragma unroll
+      for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if ((vbase + mi * 16 + r) >= p.V) g.acc[mi][ni][r] = kNegBig;
+    }
+    // where this lane's eight-entry groups go: token row; lanes of odd 16-lane rows own the second
+    // block of a pair, lanes of the upper two rows the upper eight entries of a block
+    const bool store = p.zt != nullptr && (t0 + ni * 16) < zt_cols;   // tokens past the live ones are never read
+    const uint32_t voff = (uint32_t)((ni * 16 + l15) * ldz2 + (vwave + (lq & 1) * 16 + (lq >> 1) * 8) * 2);
+    bool keep = true;
+    if (store) keep = col < p.n && p.mask[col] != 0.f;     // rows of masked tokens are not written
+    auto group_off = [&](int mp) {      // kOob when the lane's eight entries lie past V (V % 8 == 0)
+      return (keep && (vwave + (2 * mp + (lq & 1)) * 16 + (lq >> 1) * 8) < p.V) ? voff : kOob;
+    };
+    float l = 0.f, s = 0.f;
+    if (store) {
+#pragma unroll
+      for (int mp = 0; mp < G::MI / 2; ++mp) {
+        float v[2][4];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float z = g.acc[2 * mp + h][ni][r];                // CAP: t = cap(z) log2(e)
+            const float e = __builtin_amdgcn_exp2f(CAP ? z : z * kLog2e);
+            l += e;
+            s = fmaf(e, z, s);
+            v[h][r] = CAP ? e * fmaf(z * z, -kLn2Sq * inv_cap2, 1.f) : e;   // cap' = 1 - (cap(z) / cap)^2
+          }
+        const uint32_t x0 = pack_bf16(v[0][0], v[0][1]), x1 = pack_bf16(v[0][2], v[0][3]);
+        const uint32_t y0 = pack_bf16(v[1][0], v[1][1]), y1 = pack_bf16(v[1][2], v[1][3]);
+        // v_permlane16_swap: the first operand of the odd 16-lane rows <-> the second operand of the even ones
+        const auto s0 = __builtin_amdgcn_permlane16_swap(x0, y0, false, false);
+        const auto s1 = __builtin_amdgcn_permlane16_swap(x1, y1, false, false);
+        const u32x4 out = {s0[0], s1[0], s0[1], s1[1]};
+        __builtin_amdgcn_raw_buffer_store_b128(out, zrs, group_off(mp), (uint32_t)(mp * 32) * 2, 0);
+      }
+    } else {
+#pragma unroll
+      for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float z = g.acc[mi][ni][r];
+          const float e = __builtin_amdgcn_exp2f(CAP ? z : z * kLog2e);
+          l += e;
+          s = fmaf(e, z, s);
+        }
+    }
+    float lt = 0.f;
+    if (p.inv_t != 1.f) {
+      // the entropy is that of softmax(z / T) (train_modules/__init__.py:136): its own pair of sums,
+      // behind a real scalar branch so that the usual T = 1 pays nothing for it
+      asm volatile("");
+      const float kt = (CAP ? 1.f : kLog2e) * p.inv_t;
+      s = 0.f;
+#pragma unroll
+      for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float z = g.acc[mi][ni][r];
+          const float e = __builtin_amdgcn_exp2f(z * kt);
+          lt += e;
+          s = fmaf(e, z, s);
+        }
+      lt += __shfl_xor(lt, 16);
+      lt += __shfl_xor(lt, 32);
+    }
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    s += __shfl_xor(s, 16);
+    s += __shfl_xor(s, 32);
+    if (CAP) s *= kLn2;                      // sum e * cap(z) in natural units
+    if (lq == 0) {
+      const int64_t o = (int64_t)(tm * 2 + wm) * p.ld_p + col;
+      p.pl[o] = l;
+      p.ps[o] = s;
+      if (p.inv_t != 1.f) p.plt[o] = lt;
+    }
+    // the sampled token's logit: exactly one lane of one tile holds it
+    {
+      const int y = col < p.n ? clamp_target(p.targets[col], p.V) : -1;
+      const int d = y - vwave;                       // row inside the wavefront's 128
+      const bool hit = y >= 0 && d >= 0 && d < G::WM && ((d >> 2) & 3) == lq;
+      if (__any(hit)) {
+        const int flat = (d >> 4) * 4 + (d & 3);     // mi*4 + r
+        float zy = 0.f;
+#pragma unroll
+        for (int mi = 0; mi < G::MI; ++mi)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) zy = (flat == mi * 4 + r) ? g.acc[mi][ni][r] : zy;
+        if (hit) p.zy[col] = CAP ? zy * kLn2 : zy;
       }
     }
   }
@@ -405,7 +505,8 @@ template <int BM, int BN, int MODE, bool RESCUE, bool CAP>
 __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap map) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   int tm, tn, split;
-  if (RESCUE) {
+  static_assert(!(RESCUE && MODE == kStatsExp), "the rescue pass is a kStatsMax pass");
+  if constexpr (RESCUE) {
     if (__builtin_amdgcn_readfirstlane(*p.state) == 0) return;
     const int items = map.items();
     for (int item = blockIdx.x; item < items; item += gridDim.x) {
@@ -415,7 +516,8 @@ __global__ __launch_bounds__(kThreads) void k_logits_stats(LogitsArgs p, TileMap
   } else {
     if (MODE == kStatsExp && blockIdx.x == 0 && threadIdx.x == 0) *p.state = 0;
     if (!map.tile(blockIdx.x, tm, tn, split)) return;
-    logits_tile<BM, BN, MODE, CAP>(p, tm, tn, smem, threadIdx.x);
+    if constexpr (MODE == kStatsExp) logits_tile16<BM, BN, CAP>(p, tm, tn, smem, threadIdx.x);
+    else logits_tile<BM, BN, MODE, CAP>(p, tm, tn, smem, threadIdx.x);
   }
 }
 
@@ -732,7 +834,7 @@ struct DhArgs {
 
 template <int BM, int BN>
 __global__ __launch_bounds__(kThreads) void k_dhidden(DhArgs p, TileMap map) {
-  using G = GemmTN16<BM, BN, kRowK, kRowK, 1, true, false>;   // rows of dead tokens are not fetched
+  using G = GemmTN16<BM, BN, kRowK, kRowK, true, false>;   // rows of dead tokens are not fetched
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const TileMap live(live_pad(p.n_live, p.c0, p.n_pad) / BM, map.tiles_n, map.n_first, map.lgm, map.splits, map.lgs);
   int tm, tn, split;
