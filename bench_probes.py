@@ -118,8 +118,9 @@ def mfma_probe(torch, blib, dev):
     res = {"metric": "mfma_only_bf16_tflops", "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS,
            "kernel": "k_probe_mfma: 1024 workgroups x 4 wavefronts x 256 accumulators (4x4 blocks of "
                      "v_mfma_f32_32x32x16_bf16, or 8x8 blocks of v_mfma_f32_16x16x32_bf16), operands in registers, "
-                     "two operand sets alternating"}
-    for shape, sname in ((0, "32x32x16"), (1, "16x16x32")):
+                     "two operand sets alternating; 'chained': the two k-steps of a block back to back on "
+                     "its accumulator (the order of the GemmTN16 engine), otherwise the accumulators in rotation"}
+    for shape, sname in ((0, "32x32x16"), (1, "16x16x32"), (2, "16x16x32_chained")):
         for name in ("random", "zero"):
             ops = torch.randn(512 * 1024, device=dev).to(torch.bfloat16) if name == "random" \
                 else torch.zeros(512 * 1024, dtype=torch.bfloat16, device=dev)

@@ -29,7 +29,9 @@ void mj_bench_trace(void* user, int kernel_id, int phase, void* stream);
  * floats; *flop receives the flop executed.  Timed by the caller with events on `stream`; shows what
  * the matrix cores sustain under the GPU's power cap for a given operand data pattern.
  * shape 0: 4 x 4 blocks of v_mfma_f32_32x32x16_bf16 per wavefront, shape 1: 8 x 8 blocks of
- * v_mfma_f32_16x16x32_bf16 (twice the flop per iteration; *flop accounts for it). */
+ * v_mfma_f32_16x16x32_bf16 (twice the flop per iteration; *flop accounts for it), both with the
+ * accumulators in rotation; shape 2: as 1 with the two k-steps of a block issued back to back on its
+ * accumulator (the order of the GemmTN16 tile engine). */
 int mj_bench_probe_mfma(const void* operands, float* out, int workgroups, int iters, int shape, double* flop,
                         void* stream);
 

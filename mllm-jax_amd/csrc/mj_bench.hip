@@ -35,9 +35,11 @@ struct Profiler {
 namespace mj {
 
 // One workgroup = 4 wavefronts, each with the register tile of the product kernels: 4 x 4 blocks of
-// v_mfma_f32_32x32x16_bf16 (SHAPE 0) or 8 x 8 blocks of v_mfma_f32_16x16x32_bf16 (SHAPE 1), 256
+// v_mfma_f32_32x32x16_bf16 (SHAPE 0) or 8 x 8 blocks of v_mfma_f32_16x16x32_bf16 (SHAPE 1, 2), 256
 // accumulators either way.  Two operand sets alternate so that consecutive instructions never see
-// the same inputs.  Per wavefront and iteration: 2 * 16 * 32768 flop (SHAPE 0), 2 * 64 * 16384 (SHAPE 1).
+// the same inputs.  SHAPE 0, 1: the accumulators in rotation (k-step outer, blocks inner); SHAPE 2:
+// the two k-steps of a block back to back on its accumulator (the order of GemmTN16).  Per wavefront
+// and iteration: 2 * 16 * 32768 flop (SHAPE 0), 2 * 64 * 16384 (SHAPE 1, 2).
 template <int SHAPE>
 __global__ __launch_bounds__(256) void k_probe_mfma(const bf16x8* src, float* out, int iters) {
   constexpr int F = SHAPE == 0 ? 4 : 8;      // fragments per operand and k-step
@@ -84,13 +86,24 @@ __global__ __launch_bounds__(256) void k_probe_mfma(const bf16x8* src, float* ou
         for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
     // one k-step of 32 over the 8 x 8 blocks = the flop of two k-steps of 16 over 4 x 4 blocks of 32 x 32
     for (int it = 0; it < iters; ++it) {
+      if (SHAPE == 1) {
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][i], b[s][j], acc[i][j], 0, 0, 0);
+      } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i)
 #pragma unroll
-          for (int j = 0; j < 8; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][i], b[s][j], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < 8; ++j) {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[0][i], b[0][j], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[1][i], b[1][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);     // keeps the pair together
+          }
+      }
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i)
@@ -174,8 +187,9 @@ int mj_bench_probe_mfma(const void* operands, float* out, int workgroups, int it
   if (((uintptr_t)operands & 15u) != 0) return fail("probe: operands must be 16-byte aligned");
   if (shape == 0) mj::k_probe_mfma<0><<<workgroups, 256, 0, (hipStream_t)stream>>>((const mj::bf16x8*)operands, out, iters);
   else if (shape == 1) mj::k_probe_mfma<1><<<workgroups, 256, 0, (hipStream_t)stream>>>((const mj::bf16x8*)operands, out, iters);
-  else return fail("probe: shape must be 0 or 1");
-  const double per_iter = shape == 0 ? 2.0 * 16.0 * 32768.0 : 2.0 * 64.0 * 16384.0;
+  else if (shape == 2) mj::k_probe_mfma<2><<<workgroups, 256, 0, (hipStream_t)stream>>>((const mj::bf16x8*)operands, out, iters);
+  else return fail("probe: shape must be 0, 1 or 2");
+  const double per_iter = shape == 0 ? 2.0 * 16.0 * 32768.0 : 2.0 * 64.0 * 16384.0;   // shapes 1 and 2 alike
   if (flop) *flop = (double)workgroups * 4.0 * iters * per_iter;
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : fail("k_probe_mfma: %s", hipGetErrorString(e));
