@@ -552,7 +552,7 @@ struct GemmTN16 {
   static constexpr int kStageBytes = OpA::kBytes + OpB::kBytes;
   static constexpr int kLdsBytes = 2 * kStageBytes;
   static_assert(!(DEAD_A && LAY_A == kKRow) && !(DEAD_B && LAY_B == kKRow), "row masks only (row-major operands)");
-  static_assert(LPS <= 16, "the staged chunks of a slice ride on rows 1..5, two per five blocks");
+  static_assert(LPS <= 16, "three memory instructions per staged chunk in the 48 blocks of the first period");
 
   // acc[mi][ni][r]: row = mi*16 + (lane/16)*4 + r, col = ni*16 + lane%16 within the wavefront tile
   f32x4 acc[MI][NI];
@@ -577,32 +577,25 @@ struct GemmTN16 {
       b.slice_begin(slice);
     };
 
-    u32x4 staged[DEPTH][LPS];
-    auto load_one = [&](auto set, int slice, int j) {
-      constexpr int S = decltype(set)::value;
-      if (j < A_LD) staged[S][j] = a.load(slice, j);
-      else staged[S][j] = b.load(slice, j - A_LD);
+    u32x4 staged[LPS];
+    auto load_one = [&](int slice, int j) {
+      if (j < A_LD) staged[j] = a.load(slice, j);
+      else staged[j] = b.load(slice, j - A_LD);
     };
-    auto store_one = [&](auto set, int slice, int j) {
-      constexpr int S = decltype(set)::value;
+    auto store_one = [&](int slice, int j) {
       char* stage = smem + (slice & 1) * kStageBytes;
-      if (j < A_LD) a.store(stage, j, staged[S][j]);
-      else b.store(stage + OpA::kBytes, j - A_LD, staged[S][j]);
+      if (j < A_LD) a.store(stage, j, staged[j]);
+      else b.store(stage + OpA::kBytes, j - A_LD, staged[j]);
     };
-    auto store_half = [&](auto set, int slice, int j, int h) {
-      constexpr int S = decltype(set)::value;
+    auto store_half = [&](int slice, int j, int h) {
       char* stage = smem + (slice & 1) * kStageBytes;
-      if (j < A_LD) a.store_half(stage, j, staged[S][j], h);
-      else b.store_half(stage + OpA::kBytes, j - A_LD, staged[S][j], h);
+      if (j < A_LD) a.store_half(stage, j, staged[j], h);
+      else b.store_half(stage + OpA::kBytes, j - A_LD, staged[j], h);
     };
     bf16x8 fa[3][2], fb[NI][2];
     auto read_a_half = [&](int slice, int i, int ks) {
       const char* stage = smem + (slice & 1) * kStageBytes;
       fa[slot(i)][ks] = a.frag16(stage, i, ks);
-    };
-    auto read_a = [&](int slice, int i) {
-      read_a_half(slice, i, 0);
-      read_a_half(slice, i, 1);
     };
     auto read_b = [&](int slice, int j) {
       const char* stage = smem + (slice & 1) * kStageBytes + OpA::kBytes;
@@ -610,7 +603,8 @@ struct GemmTN16 {
       fb[j][1] = b.frag16(stage, j, 1);
     };
     // first: the k-step 0..31 of block (i, j); second: its k-step 32..63, on the first one's result.
-    // A block's memory instructions sit between the two.
+    // The second cannot issue before the first has gone through the matrix unit (16 cycles): a block's
+    // memory instruction sits between the two, where the wavefront would otherwise wait.
     auto first = [&](auto init, auto lead, int i, int j) {
       constexpr bool kInit = decltype(init)::value != 0, kLead = decltype(lead)::value != 0;
       (void)fa; (void)fb; (void)acc;     // named outside the assembly too, so that the lambda captures them
@@ -633,86 +627,98 @@ struct GemmTN16 {
     const int KT = (K + kBK - 1) / kBK;
     slices_begin(0);
 #pragma unroll
-    for (int j = 0; j < LPS; ++j) load_one(IntTag<0>(), 0, j);
+    for (int j = 0; j < LPS; ++j) load_one(0, j);
     slices_begin(1);
 #pragma unroll
     for (int j = 0; j < LPS; ++j) {
-      store_one(IntTag<0>(), 0, j);
-      load_one(IntTag<0>(), DEPTH, j);
+      store_one(0, j);
+      load_one(1, j);
     }
     wait_lgkmcnt0();
-    __builtin_amdgcn_s_barrier();       // slice 0 is in LDS, the next DEPTH slices are on their way to the registers
-    read_a(0, 0);
+    __builtin_amdgcn_s_barrier();       // slice 0 is in LDS, slice 1 is on its way to the registers
+    read_a_half(0, 0, 0);
+    read_a_half(0, 0, 1);
 #pragma unroll
     for (int j = 0; j < NI; ++j) read_b(0, j);
 
-    auto mem_op = [&](auto set, int kt, int q) {
-      if (q < 0) return;
-      if (q / 5 >= LPS) return;
-      if (q % 5 == 0) store_half(set, kt + 1, q / 5, 0);
-      if (q % 5 == 2) store_half(set, kt + 1, q / 5, 1);
-      if (q % 5 == 4) load_one(set, kt + 1 + DEPTH, q / 5);
+    // A period runs from the barrier inside slice s-1 to the one inside slice s: rows 6, 7 of slice
+    // s-1, then rows 0..5 of slice s: 64 blocks.  During it slice s+1 moves from the staging registers
+    // to the LDS stage that slice s-1 has just left, and slice s+2 is loaded: per 16-byte chunk two
+    // 8-byte LDS writes and one global load, each in the gap INSIDE a block (between its two matrix
+    // instructions, where 12 issue cycles are free anyway), three blocks out of four.  The first
+    // period has no rows 6, 7: its 48 blocks carry one memory instruction each.
+    auto mem_op = [&](int s, int slot, bool first_period) {
+      const int q = first_period ? slot - 16 : slot;              // 0..47 or 0..63
+      const int c = first_period ? q / 3 : q / 4, r = first_period ? q % 3 : q % 4;
+      if (q < 0 || c >= LPS) return;
+      if (r == 0) store_half(s + 1, c, 0);
+      if (r == 1) store_half(s + 1, c, 1);
+      if (r == 2) load_one(s + 2, c);
     };
-    // Row i < 6 of slice kt.  set: the staging registers that hold slice kt+1 (refilled with slice
-    // kt+1+DEPTH).
-    auto row = [&](auto init, auto settle, auto set, int kt, int i) {
+    // One block: its two matrix instructions with the period's memory instruction `slot` between them.
+    auto block = [&](auto init, auto lead, auto settle, int i, int j, int s, int slot, bool first_period) {
+      first(init, lead, i, j);
+      __builtin_amdgcn_sched_barrier(0);
+      mem_op(s, slot, first_period);
+      __builtin_amdgcn_sched_barrier(0);
+      second(settle, i, j);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // Rows 6 and 7 of slice s-1, column by column, so that the B pairs are released one per two blocks:
+    // each is re-read for slice s after its last use (behind the next column's first block; the last
+    // one inside row 0).  more: slice s exists (its fragments are read, the period's memory
+    // instructions ride along).
+    auto rows_back = [&](auto init, auto more, int s) {
+      constexpr bool kMore = decltype(more)::value != 0;
+      if (kMore) slices_begin(s + 2);   // the period's loads
 #pragma unroll
       for (int j = 0; j < NI; ++j) {
-        const int g = (i - 1) * NI + j;
-        if (i == 1 && j == 0) first(init, IntTag<1>(), i, j);
-        else first(init, IntTag<0>(), i, j);
-        __builtin_amdgcn_sched_barrier(0);
-        // the A pair of the next row, one fragment per block (row 5: of the next two rows)
-        if (j < 2) read_a_half(kt, i + 1, j);
-        if (i == 5 && (j == 2 || j == 3)) read_a_half(kt, 7, j - 2);
-        if (i == 0 && j == 2 && kt > 0) read_b(kt, NI - 1);   // the last B pair, left over by rows_back
-        // Rows 1..5 have 80 gaps (one inside each block, one behind it); chunk c takes gaps 5c, 5c+2
-        // and 5c+4: its two 8-byte halves go to the LDS, then its register is refilled (a load issued
-        // right behind the LDS write of the same registers waits until the LDS has taken them).
-        mem_op(set, kt, i == 0 ? -1 : 2 * g);
-        __builtin_amdgcn_sched_barrier(0);
-        if (j == NI - 1) second(settle, i, j);
-        else second(IntTag<0>(), i, j);
-        __builtin_amdgcn_sched_barrier(0);
-        if (i > 0 && ((2 * g + 1) % 5 == 0 || (2 * g + 1) % 5 == 2 || (2 * g + 1) % 5 == 4)) {
-          mem_op(set, kt, 2 * g + 1);
+        if (j == 0) block(init, IntTag<1>(), IntTag<0>(), MI - 2, j, s, kMore ? 2 * j : -1, false);
+        else block(init, IntTag<0>(), IntTag<0>(), MI - 2, j, s, kMore ? 2 * j : -1, false);
+        if (kMore) {
+          if (j < 2) read_a_half(s, 0, j);
+          if (j > 0) read_b(s, j - 1);
           __builtin_amdgcn_sched_barrier(0);
         }
+        if (j == NI - 1) block(init, IntTag<0>(), IntTag<1>(), MI - 1, j, s, kMore ? 2 * j + 1 : -1, false);
+        else block(init, IntTag<0>(), IntTag<0>(), MI - 1, j, s, kMore ? 2 * j + 1 : -1, false);
       }
     };
-    // Rows 6 and 7 of slice kt, column by column, so that the B pairs are released one per two blocks:
-    // each is re-read for slice kt+1 after its last use (inside the next column's first block; the
-    // last one inside row 0), behind the barrier that publishes that slice in the LDS.
-    auto rows_back = [&](auto init, int kt) {
-      wait_lgkmcnt0();                  // own reads of slice kt and writes of slice kt+1 are done
+    // Rows 0..5 of slice s; the A pair of row i+1 is read meanwhile (row 5: of rows 6 and 7).
+    auto rows_front = [&](auto init, int s, bool first_period) {
+      if (first_period) slices_begin(s + 2);
+#pragma unroll
+      for (int i = 0; i < MI - 2; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+          if (i == MI - 3 && j == NI - 1) block(init, IntTag<0>(), IntTag<1>(), i, j, s, 16 + i * NI + j, first_period);
+          else block(init, IntTag<0>(), IntTag<0>(), i, j, s, 16 + i * NI + j, first_period);
+          if (j < 2) read_a_half(s, i + 1, j);
+          if (i == 5 && (j == 2 || j == 3)) read_a_half(s, 7, j - 2);
+          if (i == 0 && j == 2 && !first_period) read_b(s, NI - 1);   // the last B pair, left over by rows_back
+          __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto publish = [&]() {
+      wait_lgkmcnt0();                  // own reads of the slice that ends and writes of the next one are done
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int j = 0; j < NI; ++j) {
-        first(init, IntTag<0>(), MI - 2, j);
-        __builtin_amdgcn_sched_barrier(0);
-        if (j < 2) read_a_half(kt + 1, 0, j);
-        if (j > 0) read_b(kt + 1, j - 1);
-        __builtin_amdgcn_sched_barrier(0);
-        second(IntTag<0>(), MI - 2, j);
-        __builtin_amdgcn_sched_barrier(0);
-        first(init, IntTag<0>(), MI - 1, j);
-        __builtin_amdgcn_sched_barrier(0);
-        second(IntTag<0>(), MI - 1, j);
-        __builtin_amdgcn_sched_barrier(0);
+    };
+    // Every accumulator is first written at exactly one place (rows 0..5: the first period; rows 6, 7:
+    // the second one, which with a single slice reads the zero-filled stage of a slice past K and
+    // starts loads that the buffer descriptors reject).
+    rows_front(IntTag<1>(), 0, true);
+    publish();
+    rows_back(IntTag<1>(), IntTag<1>(), 1);
+    if (KT > 1) {
+      rows_front(IntTag<0>(), 1, false);
+      for (int s = 2; s < KT; ++s) {
+        publish();
+        rows_back(IntTag<0>(), IntTag<1>(), s);
+        rows_front(IntTag<0>(), s, false);
       }
-    };
-    // The last iteration's row 0 multiplies the zero-filled stage of a slice past K.
-    auto iteration = [&](auto init, auto set, int kt) {
-      slices_begin(kt + 1 + DEPTH);
-#pragma unroll
-      for (int i = 1; i < MI - 2; ++i) row(init, IntTag<0>(), set, kt, i);
-      rows_back(init, kt);
-      row(IntTag<0>(), IntTag<1>(), set, kt + 1, 0);
-    };
-    row(IntTag<1>(), IntTag<0>(), IntTag<0>(), 0, 0);
-    iteration(IntTag<1>(), IntTag<0>(), 0);
-    for (int kt = 1; kt < KT; ++kt) iteration(IntTag<0>(), IntTag<0>(), kt);
+      rows_back(IntTag<0>(), IntTag<0>(), KT);
+    }
   }
 };
 
