@@ -283,17 +283,15 @@ struct KDead {
 // during slice k and written to the LDS during slice k+1 (one slice of math to land).  2: a second
 // set of staging registers; the loads of slice k+3 are issued during slice k and written during
 // slice k+2 (two slices to land) -- for shapes whose operands come from HBM on every slice.
-// DEAD_A / DEAD_B: the operand takes a mask of rows (kRowK) or k-rows (kKRow) known to be zero.
-template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK, int DEPTH = 1, bool DEAD_A = false,
-          bool DEAD_B = false, int WAVES_M = 2, int WAVES_N = 2>
+template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK, int DEPTH = 1, int WAVES_M = 2, int WAVES_N = 2>
 struct GemmTN {
   static_assert(BM % 32 == 0 && BN % 32 == 0, "tile sides are multiples of 32");
   static constexpr int kWavesM = WAVES_M, kWavesN = WAVES_N;
   static constexpr int kThreads = 64 * WAVES_M * WAVES_N;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;   // wavefront tile
   static constexpr int MI = WM / 32, NI = WN / 32;   // 32x32 blocks per wavefront
-  using OpA = Operand<BM, LAY_A, kThreads, DEAD_A>;
-  using OpB = Operand<BN, LAY_B, kThreads, DEAD_B>;
+  using OpA = Operand<BM, LAY_A, kThreads>;
+  using OpB = Operand<BN, LAY_B, kThreads>;
   static constexpr int A_LD = OpA::LD, B_LD = OpB::LD;
   static constexpr int LPS = A_LD + B_LD;            // 16-byte chunks per thread per slice
   static constexpr int kStageBytes = OpA::kBytes + OpB::kBytes;
@@ -309,37 +307,27 @@ struct GemmTN {
   // tid: the thread's index in the workgroup (a kernel that loops over tiles passes a value the
   // compiler cannot see through, so that the per-thread address arithmetic is redone per tile
   // instead of living in registers across the epilogue).
-  static constexpr bool kKDead = (DEAD_A && LAY_A == kKRow) || (DEAD_B && LAY_B == kKRow);
-  static_assert(!kKDead || (BM == 256 && BN == 256 && LAY_A == kKRow && LAY_B == kKRow && DEAD_A && DEAD_B),
-                "a k-row mask covers both operands of a 256 x 256 tile");
-
-  // dead_a / dead_b: see Operand::init and KDead (only read when DEAD_A / DEAD_B; a k-row mask is
-  // one list, passed as dead_a).
   MJ_DEV void run(const __bf16* A, int rows_a, int64_t lda, const __bf16* B, int rows_b,
-                  int64_t ldb, int K, char* smem, int tid = threadIdx.x, const uint64_t* dead_a = nullptr,
-                  const uint64_t* dead_b = nullptr) {
+                  int64_t ldb, int K, char* smem, int tid = threadIdx.x) {
     if (DEPTH == 2) {
-      run_deep(A, rows_a, lda, B, rows_b, ldb, K, smem, tid, dead_a, dead_b);
+      run_deep(A, rows_a, lda, B, rows_b, ldb, K, smem, tid);
       return;
     }
     const int wave = tid >> 6;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     OpA a;
     OpB b;
-    a.init(A, rows_a, lda, K, wm * WM, tid, dead_a);
-    b.init(B, rows_b, ldb, K, wn * WN, tid, dead_b);
-    KDead kd;
-    if (kKDead) kd.init(dead_a, K, tid);
+    a.init(A, rows_a, lda, K, wm * WM, tid);
+    b.init(B, rows_b, ldb, K, wn * WN, tid);
     auto slices_begin = [&](int slice) {
       a.slice_begin(slice);
       b.slice_begin(slice);
-      if (kKDead) kd.slice_begin(slice);
     };
 
     u32x4 staged[LPS];
     auto load_one = [&](int slice, int j) {
-      if (j < A_LD) staged[j] = kKDead ? a.load(slice, j, kd.lo, kd.hi) : a.load(slice, j);
-      else staged[j] = kKDead ? b.load(slice, j - A_LD, kd.lo, kd.hi) : b.load(slice, j - A_LD);
+      if (j < A_LD) staged[j] = a.load(slice, j);
+      else staged[j] = b.load(slice, j - A_LD);
     };
     auto store_one = [&](int slice, int j) {
       char* stage = smem + (slice & 1) * kStageBytes;
@@ -413,38 +401,29 @@ struct GemmTN {
   // (kt+1) & 1 and refills that set with slice kt+3; the loop is unrolled by two so that the set
   // index is a compile-time constant.
   MJ_DEV void run_deep(const __bf16* A, int rows_a, int64_t lda, const __bf16* B, int rows_b, int64_t ldb,
-                       int K, char* smem, int tid, const uint64_t* dead_a, const uint64_t* dead_b) {
+                       int K, char* smem, int tid) {
     const int wave = tid >> 6;
     const int wm = wave % WAVES_M, wn = wave / WAVES_M;
     OpA a;
     OpB b;
-    a.init(A, rows_a, lda, K, wm * WM, tid, dead_a);
-    b.init(B, rows_b, ldb, K, wn * WN, tid, dead_b);
-    KDead kd;
-    if (kKDead) kd.init(dead_a, K, tid);
+    a.init(A, rows_a, lda, K, wm * WM, tid);
+    b.init(B, rows_b, ldb, K, wn * WN, tid);
     auto slices_begin = [&](int slice) {
       a.slice_begin(slice);
       b.slice_begin(slice);
-      if (kKDead) kd.slice_begin(slice);
     };
 
     u32x4 staged[2][LPS];
     auto load_one = [&](auto set, int slice, int j) {
       constexpr int S = decltype(set)::value;
-      if (j < A_LD) staged[S][j] = kKDead ? a.load(slice, j, kd.lo, kd.hi) : a.load(slice, j);
-      else staged[S][j] = kKDead ? b.load(slice, j - A_LD, kd.lo, kd.hi) : b.load(slice, j - A_LD);
+      if (j < A_LD) staged[S][j] = a.load(slice, j);
+      else staged[S][j] = b.load(slice, j - A_LD);
     };
     auto store_one = [&](auto set, int slice, int j) {
       constexpr int S = decltype(set)::value;
       char* stage = smem + (slice & 1) * kStageBytes;
       if (j < A_LD) a.store(stage, j, staged[S][j]);
       else b.store(stage + OpA::kBytes, j - A_LD, staged[S][j]);
-    };
-    auto store_half = [&](auto set, int slice, int j, int h) {
-      constexpr int S = decltype(set)::value;
-      char* stage = smem + (slice & 1) * kStageBytes;
-      if (j < A_LD) a.store_half(stage, j, staged[S][j], h);
-      else b.store_half(stage + OpA::kBytes, j - A_LD, staged[S][j], h);
     };
     bf16x8 fa[2][MI], fb[2][NI];
     auto read_one = [&](int slice, int ks, int buf, int g) {
@@ -551,7 +530,9 @@ struct GemmTN16 {
   static constexpr int A_LD = OpA::LD, B_LD = OpB::LD, LPS = A_LD + B_LD;
   static constexpr int kStageBytes = OpA::kBytes + OpB::kBytes;
   static constexpr int kLdsBytes = 2 * kStageBytes;
-  static_assert(!(DEAD_A && LAY_A == kKRow) && !(DEAD_B && LAY_B == kKRow), "row masks only (row-major operands)");
+  // a mask over k-rows comes with a k-major A; it is read once and would serve a k-major B as well
+  static constexpr bool kKDead = DEAD_A && LAY_A == kKRow;
+  static_assert(!(DEAD_B && LAY_B == kKRow), "k-row masks are handed in with A");
   static_assert(LPS <= 16, "three memory instructions per staged chunk in the 48 blocks of the first period");
 
   // acc[mi][ni][r]: row = mi*16 + (lane/16)*4 + r, col = ni*16 + lane%16 within the wavefront tile
@@ -572,14 +553,17 @@ struct GemmTN16 {
     b.init(B, rows_b, ldb, K, wn * WN, tid, dead_b);
     a.init16(wm * WM, tid);
     b.init16(wn * WN, tid);
-    auto slices_begin = [&](int slice) {
+    KDead kd;
+    if (kKDead) kd.init(dead_a, K, tid);
+    auto slices_begin = [&](int slice) {     // in slice order: the mask word of the next slice is requested here
       a.slice_begin(slice);
       b.slice_begin(slice);
+      if (kKDead) kd.slice_begin(slice);
     };
 
     u32x4 staged[LPS];
     auto load_one = [&](int slice, int j) {
-      if (j < A_LD) staged[j] = a.load(slice, j);
+      if (j < A_LD) staged[j] = kKDead ? a.load(slice, j, kd.lo, kd.hi) : a.load(slice, j);
       else staged[j] = b.load(slice, j - A_LD);
     };
     auto store_one = [&](int slice, int j) {

@@ -282,11 +282,6 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
         Timed t(MJ_GRPO_K_FINALIZE, st);
         mj::k_finalize<mj::kStatsExp><<<n_pad / mj::kFinTokens, mj::kFinTokens * mj::kFinSlices, 0, st>>>(f);
       }
-      if (bwd) {
-        const int64_t work = (int64_t)nc * (H / 8);
-        Timed t(MJ_GRPO_K_SCALE_HIDDEN, st);
-        mj::k_scale_hidden<<<(unsigned)((work + 255) / 256), 256, 0, st>>>((const uint16_t*)hid_c, ld_hid, rs, nc, H, hs);
-      }
       // the rescue: the same chunk with a running maximum; every workgroup leaves at once unless the
       // range check in k_finalize failed
       Timed t(MJ_GRPO_K_RESCUE, st);
@@ -330,10 +325,17 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
                                                                            h.ld_dh, rs, state, h.dv, h.wv);
       }
 
+      // the token-side operand of the dW product, k-contiguous: (rs * hidden)^T while the 16-bit matrix
+      // holds E, hidden^T once it holds dZ (the state word is final by now)
+      {
+        Timed t(MJ_GRPO_K_SCALE_HIDDEN, st);
+        mj::k_scale_hidden<<<dim3((unsigned)(n_pad / 64), (unsigned)((H + 63) / 64)), 256, 0, st>>>(
+            (const uint16_t*)hid_c, ld_hid, rs, state, nc, n_pad, H, hs);
+      }
       mj::DwArgs w;
-      w.dzt = (const __bf16*)zt; w.hid = hid_c; w.hs = (const __bf16*)hs; w.ld_z = p.ld_z; w.ld_hid = ld_hid;
+      w.dzt = (const __bf16*)zt; w.ht = (const __bf16*)hs; w.ld_z = p.ld_z;
       w.H = H; w.V = V; w.n = nc;
-      w.dw = d_w; w.ld_dw = d->ld_w; w.n_live = n_live; w.c0 = (int)c0; w.state = state; w.dead = dead;
+      w.dw = d_w; w.ld_dw = d->ld_w; w.n_live = n_live; w.c0 = (int)c0; w.dead = dead;
       w.accumulate = (c0 > 0 || (d->flags & MJ_GRPO_FLAG_DW_ACCUMULATE)) ? 1 : 0;
       const mj::TileMap mw = mj::TileMap::pick_shape((V + BM - 1) / BM, (H + BN - 1) / BN, 0, 1);
       {

@@ -675,21 +675,38 @@ __global__ __launch_bounds__(kFinTokens * kFinSlices) void k_finalize(FinalizeAr
   }
 }
 
-// rs[t] * hidden[t, :] in bf16: the token-side operand of the dW product when the 16-bit matrix
-// holds E (one thread = 8 columns)
-__global__ __launch_bounds__(256) void k_scale_hidden(const uint16_t* hid, int64_t ld_hid, const float* rs, int n,
-                                                      int H, uint16_t* hs) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int h8 = H >> 3;
-  if (i >= (int64_t)n * h8) return;
-  const int row = (int)(i / h8), c = (int)(i % h8) * 8;
-  const float r = rs[row];
-  const u32x4 in = *(const u32x4*)(hid + (int64_t)row * ld_hid + c);
-  u32x4 out;
+// The token-side operand of the dW product, k-contiguous: ht[h, t] = c_t * hidden[t, h] as a
+// [H, n_pad] bf16 matrix, c_t = rs[t] while the 16-bit matrix holds E and 1 once it holds dZ; zeros
+// for t >= n.  One workgroup transposes 64 tokens x 64 columns through the LDS.
+__global__ __launch_bounds__(256) void k_scale_hidden(const uint16_t* hid, int64_t ld_hid, const float* rs,
+                                                  const int* state, int n, int n_pad, int H, uint16_t* ht) {
+  __shared__ uint16_t tile[64][72];            // [token][column]; 144-byte rows keep the 16-byte writes aligned
+  const int t0 = blockIdx.x * 64, h0 = blockIdx.y * 64;
+  const bool scaled = *state == 0;
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
-    out[j] = pack_bf16(r * __uint_as_float(in[j] << 16), r * __uint_as_float(in[j] & 0xffff0000u));
-  *(u32x4*)(hs + (int64_t)row * H + c) = out;
+  for (int i = 0; i < 2; ++i) {
+    const int id = threadIdx.x + 256 * i, row = id >> 3, c = (id & 7) * 8;
+    const int t = t0 + row;
+    u32x4 out = {0u, 0u, 0u, 0u};
+    if (t < n && h0 + c < H) {
+      const float r = scaled ? rs[t] : 1.f;
+      const u32x4 in = *(const u32x4*)(hid + (int64_t)t * ld_hid + h0 + c);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        out[j] = pack_bf16(r * __uint_as_float(in[j] << 16), r * __uint_as_float(in[j] & 0xffff0000u));
+    }
+    *(u32x4*)&tile[row][c] = out;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int id = threadIdx.x + 256 * i, h = id >> 3, c = (id & 7) * 8;
+    if (h0 + h >= H) continue;
+    u32x4 out;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[j] = (uint32_t)tile[c + 2 * j][h] | ((uint32_t)tile[c + 2 * j + 1][h] << 16);
+    *(u32x4*)(ht + (int64_t)(h0 + h) * n_pad + t0 + c) = out;
+  }
 }
 
 // dloss/dlogp from a saved forward (separate backward entry point)
@@ -908,44 +925,38 @@ __global__ __launch_bounds__(256) void k_dhidden_reduce(const float* part, int s
 
 struct DwArgs {
   const __bf16* dzt;   // [n, ld_z] E or dZ of the chunk
-  const __bf16* hid;   // chunk origin [n, ld_hid]
-  const __bf16* hs;    // [n, H]: rs * hidden, the token-side operand while state == 0
-  int64_t ld_z, ld_hid;
+  const __bf16* ht;    // [H, n_pad]: k_scale_hidden's matrix, the token-side operand
+  int64_t ld_z;
   int H, V, n;         // n = tokens of the chunk
   void* dw;            // [H, ld_dw]: f32, or bf16 in the BF16OUT kernel
   int64_t ld_dw;
   int accumulate;
   const int* n_live;   // see live_pad
   int c0;
-  const int* state;
   const uint64_t* dead;   // [n_pad / 64] dead-token bits of the chunk
 };
 
-// Tile of dW^T: rows = vocab (MFMA row direction), columns = hidden (lanes).  A lane's four
-// consecutive accumulator rows are four consecutive floats of one dW row: 16-byte accesses.
-// Both operands are token-major in memory, so both go through the transposing LDS read.
-// BF16OUT: dW is a bf16 matrix; two lanes exchange halves (store_rows8) so that each writes eight
-// consecutive entries of one row, and an accumulating call adds in fp32 and rounds once.
+// Tile of dW^T: rows = vocab (MFMA row direction), columns = hidden (lanes), on the chained
+// 16 x 16 x 32 engine (GemmTN16).  The token-side operand is k_scale_hidden's [H, n_pad] matrix, so
+// only E / dZ (token-major in memory) goes through the transposing LDS read; the token rows of dead
+// tokens are not fetched.  A lane's four accumulator rows of a block are four consecutive entries of
+// one dW row: one 16-byte access per block in float32; in bf16 the lanes l and l + 16 exchange, two
+// blocks at a time, so that each owns eight consecutive entries (an accumulating call adds in fp32
+// and rounds once).
 template <int BM, int BN, bool BF16OUT>
 __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
-  // two slices in flight: measured 2-3% faster here, not in the other products; the token rows of
-  // dead tokens (k-rows of both operands) are not fetched
-  using G = GemmTN<BM, BN, kKRow, kKRow, 2, true, true>;
+  using G = GemmTN16<BM, BN, kKRow, kRowK, true, false>;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   int tm, tn, split;
   if (!map.tile(blockIdx.x, tm, tn, split)) return;
   const int m0 = tm * BM, n0 = tn * BN;
   G g;
-  const int kn = min(p.n, live_pad(p.n_live, p.c0, (p.n + 255) & ~255));   // tokens past the live ones have dZ = 0
-  const bool scaled = __builtin_amdgcn_readfirstlane(*p.state) == 0;
-  const __bf16* tok = scaled ? p.hs : p.hid;
-  const int64_t ld_tok = scaled ? (int64_t)p.H : p.ld_hid;
-  g.run(p.dzt + m0, p.V - m0, p.ld_z, tok + n0, p.H - n0, ld_tok, kn, smem, threadIdx.x, p.dead, p.dead);
+  const int n_pad = (p.n + 255) & ~255;
+  const int kn = min(p.n, live_pad(p.n_live, p.c0, n_pad));   // tokens past the live ones have dZ = 0
+  g.run(p.dzt + m0, p.V - m0, p.ld_z, p.ht + (int64_t)n0 * n_pad, p.H - n0, n_pad, kn, smem, threadIdx.x, p.dead);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keeps descriptors in SGPRs
-  const int wm = wave & 1, wn = wave >> 1, l31 = lane & 31, lhi = lane >> 5;
-  // dW rows of this wavefront's 128 hidden columns, starting at its first vocab column; a lane's
-  // address is (its hidden row) * ld + (its 4-float group), the vocab block is the scalar offset.
+  const int wm = wave & 1, wn = wave >> 1, l15 = lane & 15, lq = lane >> 4;
   const int h0 = n0 + wn * G::WN, v0 = m0 + wm * G::WM;
   const int hrows = min(max(p.H - h0, 0), G::WN);
   const int vleft = p.V - v0;                            // V % 8 == 0: groups of 4 or 8 are in or out together
@@ -953,42 +964,39 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
     const uint32_t ld2 = (uint32_t)p.ld_dw * 2;
     const __amdgpu_buffer_rsrc_t rs =
         make_rsrc_wave((uint16_t*)p.dw + (int64_t)h0 * p.ld_dw + v0, (int64_t)hrows * ld2 - (int64_t)v0 * 2);
+    const int vlane = (lq & 1) * 16 + (lq >> 1) * 8;     // the lane's eight entries of a block pair's 32
 #pragma unroll
     for (int ni = 0; ni < G::NI; ++ni) {
-      const uint32_t lane_off = (uint32_t)((ni * 32 + l31) * ld2 + lhi * 16);   // the lane's 16 of a pair's 32 bytes
-      u32x4 old[G::MI][2];
-      if (p.accumulate) {                     // all loads of this column block before its first store
+      const uint32_t lane_off = (uint32_t)((ni * 16 + l15) * ld2 + vlane * 2);
+      u32x4 old[G::MI / 2];
+      if (p.accumulate) {                     // all loads of this column of blocks before its first store
 #pragma unroll
-        for (int mi = 0; mi < G::MI; ++mi)
-#pragma unroll
-          for (int qp = 0; qp < 2; ++qp) {
-            const int vv = mi * 32 + qp * 16;
-            old[mi][qp] = __builtin_amdgcn_raw_buffer_load_b128(rs, (vv + lhi * 8) < vleft ? lane_off : kOob,
-                                                                (uint32_t)vv * 2, 0);
-          }
+        for (int mp = 0; mp < G::MI / 2; ++mp)
+          old[mp] = __builtin_amdgcn_raw_buffer_load_b128(rs, (mp * 32 + vlane) < vleft ? lane_off : kOob,
+                                                          (uint32_t)(mp * 32) * 2, 0);
       }
 #pragma unroll
-      for (int mi = 0; mi < G::MI; ++mi)
+      for (int mp = 0; mp < G::MI / 2; ++mp) {
+        float v[8];
 #pragma unroll
-        for (int qp = 0; qp < 2; ++qp) {
-          const int vv = mi * 32 + qp * 16;
-          float v[8];
-#pragma unroll
-          for (int j = 0; j < 8; ++j) v[j] = g.acc[mi][ni][qp * 8 + j];
-          if (p.accumulate) {
-            // undo the exchange of store_rows8 on what is in memory (the exchange is its own inverse)
-            const u32x4 o = old[mi][qp];
-            const auto s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
-            const auto s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
-            const uint32_t w[4] = {s0[0], s1[0], s0[1], s1[1]};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              v[2 * j] += __uint_as_float(w[j] << 16);
-              v[2 * j + 1] += __uint_as_float(w[j] & 0xffff0000u);
-            }
-          }
-          store_rows8<false>(v, rs, (vv + lhi * 8) < vleft ? lane_off : kOob, (uint32_t)vv * 2);
+        for (int r = 0; r < 4; ++r) {
+          // v_permlane16_swap: the first operand of the odd 16-lane rows <-> the second operand of the even ones
+          const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(g.acc[2 * mp][ni][r]),
+                                                           __float_as_uint(g.acc[2 * mp + 1][ni][r]), false, false);
+          v[r] = __uint_as_float(sw[0]);
+          v[4 + r] = __uint_as_float(sw[1]);
         }
+        if (p.accumulate) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            v[2 * j] += __uint_as_float(old[mp][j] << 16);
+            v[2 * j + 1] += __uint_as_float(old[mp][j] & 0xffff0000u);
+          }
+        }
+        const u32x4 out = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
+        __builtin_amdgcn_raw_buffer_store_b128(out, rs, (mp * 32 + vlane) < vleft ? lane_off : kOob,
+                                               (uint32_t)(mp * 32) * 2, 0);
+      }
     }
     return;
   }
@@ -997,31 +1005,18 @@ __global__ __launch_bounds__(kThreads) void k_dw(DwArgs p, TileMap map) {
       make_rsrc_wave((float*)p.dw + (int64_t)h0 * p.ld_dw + v0, (int64_t)hrows * ld4 - (int64_t)v0 * 4);
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
-    const uint32_t lane_off = (uint32_t)((ni * 32 + l31) * ld4 + lhi * 16);
+    const uint32_t lane_off = (uint32_t)((ni * 16 + l15) * ld4 + lq * 16);
+    // when accumulating, the eight loads of this column of blocks are issued before the first store (a
+    // store between two loads would order the second behind it: one memory round trip per 16 bytes)
+    f32x4 a[G::MI];
 #pragma unroll
-    for (int mh = 0; mh < G::MI; mh += 2) {
-      // when accumulating, the eight loads of this half are issued before the first store (a store
-      // between two loads would order the second behind it: one memory round trip per 16 bytes)
-      f32x4 a[2][4];
-#pragma unroll
-      for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int vv = (mh + mi) * 32 + q * 8;
-          if (p.accumulate) a[mi][q] = load_b128(rs, (vv + lhi * 4) < vleft ? lane_off : kOob, (uint32_t)vv * 4);
-          else a[mi][q] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-      for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int vv = (mh + mi) * 32 + q * 8;
-          const uint32_t voff = (vv + lhi * 4) < vleft ? lane_off : kOob;
-          const f32x4 c = {g.acc[mh + mi][ni][q * 4], g.acc[mh + mi][ni][q * 4 + 1], g.acc[mh + mi][ni][q * 4 + 2],
-                           g.acc[mh + mi][ni][q * 4 + 3]};
-          store_b128(c + a[mi][q], rs, voff, (uint32_t)vv * 4);
-        }
+    for (int mi = 0; mi < G::MI; ++mi) {
+      if (p.accumulate) a[mi] = load_b128(rs, (mi * 16 + lq * 4) < vleft ? lane_off : kOob, (uint32_t)(mi * 16) * 4);
+      else a[mi] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+#pragma unroll
+    for (int mi = 0; mi < G::MI; ++mi)
+      store_b128(g.acc[mi][ni] + a[mi], rs, (mi * 16 + lq * 4) < vleft ? lane_off : kOob, (uint32_t)(mi * 16) * 4);
   }
 }
 
