@@ -357,6 +357,17 @@ MJ_DEV void logits_tile16(const LogitsArgs& p, int tm, int tn, char* smem, int t
   const int trows = min(max(p.n - t0, 0), G::WN);
   const __amdgpu_buffer_rsrc_t zrs =
       make_rsrc_wave(p.zt == nullptr ? nullptr : p.zt + (int64_t)t0 * p.ld_z, (int64_t)trows * ldz2);
+  // the per-token inputs of all eight block columns, requested together: inside the loop each load
+  // would wait behind the stores of the column before it (the compiler cannot tell that they do not
+  // overlap), one memory round trip per column
+  float mk[G::NI];
+  int tg[G::NI];
+#pragma unroll
+  for (int ni = 0; ni < G::NI; ++ni) {
+    const int col = t0 + ni * 16 + l15;
+    mk[ni] = col < p.n ? p.mask[col] : 0.f;
+    tg[ni] = col < p.n ? clamp_target(p.targets[col], p.V) : -1;
+  }
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
     const int col = t0 + ni * 16 + l15;
@@ -404,7 +415,7 @@ MJ_DEV void logits_tile16(const LogitsArgs& p, int tm, int tn, char* smem, int t
     const bool store = p.zt != nullptr && (t0 + ni * 16) < zt_cols;   // tokens past the live ones are never read
     const uint32_t voff = (uint32_t)((ni * 16 + l15) * ldz2 + (vwave + (lq & 1) * 16 + (lq >> 1) * 8) * 2);
     bool keep = true;
-    if (store) keep = col < p.n && p.mask[col] != 0.f;     // rows of masked tokens are not written
+    if (store) keep = mk[ni] != 0.f;                        // rows of masked tokens are not written
     auto group_off = [&](int mp) {      // kOob when the lane's eight entries lie past V (V % 8 == 0)
       return (keep && (vwave + (2 * mp + (lq & 1)) * 16 + (lq >> 1) * 8) < p.V) ? voff : kOob;
     };
@@ -474,7 +485,7 @@ MJ_DEV void logits_tile16(const LogitsArgs& p, int tm, int tn, char* smem, int t
     }
     // the sampled token's logit: exactly one lane of one tile holds it
     {
-      const int y = col < p.n ? clamp_target(p.targets[col], p.V) : -1;
+      const int y = tg[ni];
       const int d = y - vwave;                       // row inside the wavefront's 128
       const bool hit = y >= 0 && d >= 0 && d < G::WM && ((d >> 2) & 3) == lq;
       if (__any(hit)) {
