@@ -25,8 +25,8 @@ PEAK_HBM_GBS = 8000.0
 # a plain 1 GiB device copy (x2.00 fetch, x1.00 write); summary in profiles/.  Keyed by
 # (config index, kernel); None for workloads that were not counted.
 MEASURED_TRAFFIC_BYTES = {          # default chunk (one launch of each kernel per step at configs 0-2 and 4)
-    (0, "k_logits_stats"): 0.40e9, (0, "k_dhidden"): 0.42e9, (0, "k_dw"): 0.68e9,
-    (2, "k_logits_stats"): 30.40e9, (2, "k_dhidden"): 36.60e9, (2, "k_dw"): 19.91e9,
+    (0, "k_logits_stats"): 0.40e9, (0, "k_dhidden"): 0.42e9, (0, "k_dw"): 0.71e9,
+    (2, "k_logits_stats"): 29.82e9, (2, "k_dhidden"): 26.12e9, (2, "k_dw"): 27.59e9,
 }
 TRAFFIC_SOURCE = {0: "profiles/cfg0_qwen05b_fused_fwd_bwd.txt", 2: "profiles/cfg2_qwen7b_fused_fwd_bwd.txt"}
 
