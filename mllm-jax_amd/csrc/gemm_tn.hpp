@@ -2,10 +2,11 @@
 //
 // C[M,N] (fp32 accumulators) = sum_k A(m,k) * B(n,k).  One workgroup of WAVES_M x WAVES_N
 // wavefronts owns a BM x BN tile; each wavefront owns (BM/WAVES_M) x (BN/WAVES_N) as a grid of
-// 32x32 MFMA blocks (v_mfma_f32_32x32x16_bf16).
+// 32x32 MFMA blocks (v_mfma_f32_32x32x16_bf16; GemmTN) or of 16x16 blocks
+// (v_mfma_f32_16x16x32_bf16 with the two k-steps of a block chained; GemmTN16, further down).
 //
-// Each operand may live in memory in either of two layouts, so no operand ever needs a
-// transposed copy:
+// Each operand may live in memory in either of two layouts, so a product can read its operands
+// where they are:
 //   kRowK : X[row][k], k contiguous  -- LDS image 128 bytes per tile row, MFMA fragments come
 //           out with one ds_read_b128 per lane;
 //   kKRow : X[k][row], rows contiguous -- LDS image 64 k-rows of 2*ROWS bytes, MFMA fragments

@@ -10,6 +10,8 @@
 //                     one-hot patch.
 //   k_dhidden       : dHidden[n,H] = rowscale * (E or dZ) * W^T, optionally split over the vocab into
 //                     fp32 partial sums that k_dhidden_reduce adds up.
+//   k_scale_hidden  : (rs * hidden)^T, or hidden^T behind a kStatsMax pass: the token-side operand of
+//                     the dW product with the tokens contiguous, [H, n_pad] bf16.
 //   k_dw            : dW^T tile [vocab x hidden] = (E or dZ)^T * (rs * hidden or hidden), written /
 //                     accumulated into dW[H,V] with 16-byte accesses.
 //   k_dz            : only behind a kStatsMax pass: in place, logits -> dZ (bf16).
