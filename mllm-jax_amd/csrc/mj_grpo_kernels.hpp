@@ -334,6 +334,16 @@ MJ_DEV void logits_tile(const LogitsArgs& p, int tm, int tn, char* smem, int tid
   }
 }
 
+// Sum of x over the four 16-lane rows of a wavefront, in every lane, without a trip through the LDS
+// crossbar: v_permlane16_swap pairs the rows (0,1) and (2,3), v_permlane32_swap the two halves.
+MJ_DEV float sum_rows16(float x) {
+  const uint32_t a = __float_as_uint(x);
+  const auto p = __builtin_amdgcn_permlane16_swap(a, a, false, false);
+  const uint32_t b = __float_as_uint(__uint_as_float(p[0]) + __uint_as_float(p[1]));
+  const auto q = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  return __uint_as_float(q[0]) + __uint_as_float(q[1]);
+}
+
 // The kStatsExp tile on the chained 16 x 16 x 32 engine (GemmTN16).  A lane holds, for the token
 // ni*16 + lane%16, the four vocab rows mi*16 + (lane/16)*4 + 0..3 of each of the eight blocks mi.
 // Two blocks at a time, the lanes l and l + 16 exchange one packed half (v_permlane16_swap) so that
@@ -471,13 +481,10 @@ MJ_DEV void logits_tile16(const LogitsArgs& p, int tm, int tn, char* smem, int t
           lt += e;
           s = fmaf(e, z, s);
         }
-      lt += __shfl_xor(lt, 16);
-      lt += __shfl_xor(lt, 32);
+      lt = sum_rows16(lt);
     }
-    l += __shfl_xor(l, 16);
-    l += __shfl_xor(l, 32);
-    s += __shfl_xor(s, 16);
-    s += __shfl_xor(s, 32);
+    l = sum_rows16(l);
+    s = sum_rows16(s);
     if (CAP) s *= kLn2;                      // sum e * cap(z) in natural units
     if (lq == 0) {
       const int64_t o = (int64_t)(tm * 2 + wm) * p.ld_p + col;
