@@ -68,7 +68,7 @@ int enable_lds(K kernel) {
   if (slot == nullptr) return fail(MJ_GRPO_ERR_UNSUPPORTED, "internal: more tile kernels than table slots");
   if (slot->fn == (const void*)kernel && slot->dev[dev]) return MJ_GRPO_OK;
   e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                          mj::GemmTN<BM, BN>::kLdsBytes);
+                          mj::GemmTN<BM, BN>::kLdsBytes + mj::kTileExtraLds);
   if (e != hipSuccess) return fail(MJ_GRPO_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   slot->fn = (const void*)kernel;
   slot->dev[dev] = true;
@@ -135,7 +135,7 @@ int run(Mode mode, const MjGrpoDesc* d, const void* hidden, const void* lm_head,
   uint16_t* zt = (uint16_t*)(ws + p.zt);
   float* part = (float*)(ws + p.part);
   const float gscale = d->grad_loss_scale;
-  const size_t lds = mj::GemmTN<BM, BN>::kLdsBytes;
+  const size_t lds = mj::GemmTN<BM, BN>::kLdsBytes + mj::kTileExtraLds;   // two stages + the epilogue's hand-over
 
   // Which statistics the logits epilogue keeps (mj::StatsMode): sums of exp(z) without a running
   // maximum plus E = exp(z) for the backward -- with a kStatsMax rescue pass enqueued behind it that

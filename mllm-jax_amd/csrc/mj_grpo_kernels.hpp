@@ -348,12 +348,26 @@ MJ_DEV float sum_rows16(float x) {
 // ni*16 + lane%16, the four vocab rows mi*16 + (lane/16)*4 + 0..3 of each of the eight blocks mi.
 // Two blocks at a time, the lanes l and l + 16 exchange one packed half (v_permlane16_swap) so that
 // each owns eight CONSECUTIVE vocab entries of one block and stores them with one 16-byte access.
+// The per-token inputs of the epilogue (mask, sampled token) are requested before the k loop, one
+// token per thread, and handed to the lanes that need them through kTileExtraLds bytes of LDS behind
+// the two stages: requested in the epilogue they cost a memory round trip per tile (2.6 us of a
+// tile's 95 at 16384 x 3584 x 152064).
+constexpr int kTileExtraLds = 2048;
 template <int BM, int BN, bool CAP>
 MJ_DEV void logits_tile16(const LogitsArgs& p, int tm, int tn, char* smem, int tid) {
   using G = GemmTN16<BM, BN, kKRow, kRowK>;
+  static_assert(BN == kThreads, "one token of the tile per thread");
   const int m0 = tm * BM, n0 = tn * BN;
+  const int tok = n0 + tid;
+  const float mask_t = tok < p.n ? p.mask[tok] : 0.f;
+  const int target_t = tok < p.n ? clamp_target(p.targets[tok], p.V) : -1;
   G g;
   g.run(p.w + m0, p.V - m0, p.ld_w, p.hid + (int64_t)n0 * p.ld_hid, p.n - n0, p.ld_hid, p.H, smem, tid);
+  float* tile_mask = (float*)(smem + G::kLdsBytes);
+  int* tile_target = (int*)(tile_mask + BN);
+  tile_mask[tid] = mask_t;
+  tile_target[tid] = target_t;
+  __syncthreads();
 
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps descriptors in SGPRs
@@ -369,16 +383,12 @@ MJ_DEV void logits_tile16(const LogitsArgs& p, int tm, int tn, char* smem, int t
   const int trows = min(max(p.n - t0, 0), G::WN);
   const __amdgpu_buffer_rsrc_t zrs =
       make_rsrc_wave(p.zt == nullptr ? nullptr : p.zt + (int64_t)t0 * p.ld_z, (int64_t)trows * ldz2);
-  // the per-token inputs of all eight block columns, requested together: inside the loop each load
-  // would wait behind the stores of the column before it (the compiler cannot tell that they do not
-  // overlap), one memory round trip per column
   float mk[G::NI];
   int tg[G::NI];
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
-    const int col = t0 + ni * 16 + l15;
-    mk[ni] = col < p.n ? p.mask[col] : 0.f;
-    tg[ni] = col < p.n ? clamp_target(p.targets[col], p.V) : -1;
+    mk[ni] = tile_mask[wn * G::WN + ni * 16 + l15];
+    tg[ni] = tile_target[wn * G::WN + ni * 16 + l15];
   }
 #pragma unroll
   for (int ni = 0; ni < G::NI; ++ni) {
