@@ -505,9 +505,10 @@ struct GemmTN {
 // registers (8 x 2 fragments); the A fragments of row i + 1 are read while row i computes (three
 // register pairs in rotation); the last two rows are walked column by column and each B fragment
 // pair is re-read for the next slice after its last use.  One barrier per slice, before those two
-// rows; the LDS writes of slice k + 1 and the global loads of slice k + 1 + DEPTH ride on rows 1..5.
-// An iteration of the loop runs from row 1 of a slice to row 0 of the next one, so that at its end
-// the youngest LDS reads are a row's time old (the compiler drains the LDS counter at a loop's top).
+// rows; the loop body runs from that barrier to the next one (a period, see run()) and carries the LDS
+// writes of the next slice and the global loads of the one after it, one slice in flight between
+// global memory and the LDS (a ring of 24 staging registers with one and a half slices in flight
+// measured 7 % slower: more requests in flight only lengthen each one).
 //
 // The matrix instructions are written as assembly so that the result register IS the accumulator
 // operand: with all 256 accumulation registers taken the register allocator otherwise routes some
@@ -515,14 +516,13 @@ struct GemmTN {
 // 0, so nothing but these instructions ever writes an accumulator.  The compiler does not see matrix
 // instructions inside the assembly, so the wait states it would put between one of them and an
 // ordinary instruction that touches an accumulator (7 behind a four-pass instruction, 2 in front)
-// are spelled out where such an instruction can follow or precede: behind the blocks of an
-// iteration's last row (loop exit; copies on the back edge, should the allocator ever make any) and
-// in front of its first block.  They cost nothing: a block keeps the matrix unit busy for 32 cycles.
+// are spelled out where such an instruction can follow or precede: behind the last block of a period
+// and of the last two rows (loop exit; copies on the back edge, should the allocator ever make any)
+// and in front of a period's first block.  They cost nothing: a block keeps the matrix unit busy for
+// 32 cycles.
 template <int BM, int BN, int LAY_A = kRowK, int LAY_B = kRowK, bool DEAD_A = false, bool DEAD_B = false>
 struct GemmTN16 {
   static_assert(BM == 256 && BN == 256, "four wavefronts of 128 x 128");
-  static constexpr int DEPTH = 1;   // slices in flight between global memory and the LDS (a second set of
-                                    // staging registers, two slices in flight, measured no faster here)
   static constexpr int kThreads = 256;
   static constexpr int WM = 128, WN = 128;
   static constexpr int MI = 8, NI = 8;               // 16 x 16 blocks per wavefront
